@@ -206,6 +206,75 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+# ---------------------------------------------------------------------------------------------------------
+# libhydra_mix.so (include/hydra_mix.h): multi-stream residuals, token shift, gated results, tanh GELU, attention over
+# a paged latent cache.  A library of its own, so that a model that needs only these builds only these (`make mix`).
+# ---------------------------------------------------------------------------------------------------------
+MIX_LIB_PATH = os.environ.get("HX_MIX_LIB_PATH") or os.path.join(_HERE, "lib", "libhydra_mix.so")
+HXM_ABI_VERSION = 1
+HXM_MAX_STREAMS = 8
+HXM_MAX_LATENT = 512
+
+
+class hxm_latent_attn_args(ctypes.Structure):
+    _fields_ = [
+        ("out", c_void_p), ("q", c_void_p), ("cache", c_void_p), ("gate_pre", c_void_p),
+        ("tok_seq", c_void_p), ("positions", c_void_p), ("q_cu", c_void_p), ("block_table", c_void_p),
+        ("cu_block_lens", c_void_p),
+        ("q_token_stride", c_int64), ("q_head_stride", c_int64), ("out_token_stride", c_int64),
+        ("out_head_stride", c_int64), ("gate_stride", c_int64), ("cache_block_stride", c_int64),
+        ("cache_row_stride", c_int64),
+        ("n_tokens", c_int32), ("n_seq", c_int32), ("n_heads", c_int32), ("kv_rank", c_int32), ("block_size", c_int32),
+        ("window", c_int32), ("max_q_len", c_int32), ("scale", c_float), ("dtype", c_int32),
+    ]
+
+
+_MIX_SIGNATURES = {
+    "hxm_abi_version": (c_int, []),
+    "hxm_last_hip_error": (c_int, []),
+    "hxm_stream_embed": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_float, c_int64, c_int32, c_int64, c_int64, c_int, c_void_p]),
+    "hxm_stream_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_float, c_void_p, c_int64, c_int32, c_int64, c_void_p,
+                                c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
+    "hxm_stream_update": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int32,
+                                  c_int64, c_int, c_void_p]),
+    "hxm_gelu_tanh_and_mul": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "hxm_latent_norm_cache": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_void_p,
+                                      c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int, c_void_p]),
+    "hxm_latent_attention": (c_int, [POINTER(hxm_latent_attn_args), c_void_p]),
+}
+
+_mix = None
+_STATUS_TEXT = {-1: "dtype not supported", -2: "size / divisibility constraint violated", -3: "layout unsupported",
+                -4: "required pointer is NULL", -5: "not implemented", -6: "workspace too small", -7: "a HIP runtime call failed"}
+
+
+def mix_lib() -> ctypes.CDLL:
+    """Open libhydra_mix.so once and type every entry point.  No fallback: a missing library raises."""
+    global _mix
+    if _mix is None:
+        if not os.path.exists(MIX_LIB_PATH):
+            raise HydraHipError(f"{MIX_LIB_PATH} is missing: build it with `make -C hydrainfer_amd/csrc mix`. "
+                                "There is no fallback path.")
+        handle = ctypes.CDLL(MIX_LIB_PATH)
+        for name, (restype, argtypes) in _MIX_SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        if handle.hxm_abi_version() != HXM_ABI_VERSION:
+            raise HydraHipError(f"libhydra_mix.so ABI version {handle.hxm_abi_version()} != {HXM_ABI_VERSION} of this binding: "
+                                "rebuild with `make -C hydrainfer_amd/csrc mix`")
+        _mix = handle
+    return _mix
+
+
+def mix_check(status: int, what: str) -> None:
+    if status != 0:
+        msg = _STATUS_TEXT.get(status, f"status {status}")
+        if status == -7:
+            msg += f" (hipError_t {mix_lib().hxm_last_hip_error()})"
+        raise HydraHipError(f"{what}: {msg}")
+
+
 def exported_symbols():
     return sorted(_SIGNATURES)
 

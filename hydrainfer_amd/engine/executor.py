@@ -64,8 +64,9 @@ class DecodeCohort:
 
 class BatchFillExecutor:
     def __init__(self, language_model, kv_cache_block_manager, image_cache_block_manager,
-                 dtype: torch.dtype, device: torch.device, graph_decoder=None):
-        self.language_model = language_model            # LlavaLanguageModel
+                 dtype: torch.dtype, device: torch.device, graph_decoder=None, state_manager=None):
+        self.state_manager = state_manager              # memory.state_slots.StateSlotManager of a model with per-sequence rows
+        self.language_model = language_model            # LlavaLanguageModel / TextLanguageModel
         lm = language_model.language_model
         self.shape = lm.shape
         self.kv_manager, self.image_manager = kv_cache_block_manager, image_cache_block_manager
@@ -308,7 +309,8 @@ class BatchFillExecutor:
         sh = self.shape
         builder = LanguageModelParametersBuilder(
             self.image_manager, self.kv_manager, sh.num_hidden_layers, sh.num_attention_heads,
-            sh.num_key_value_heads, sh.head_dim, self.language_model.image_token_id, self.dtype, self.device)
+            sh.num_key_value_heads, sh.head_dim, self.language_model.image_token_id, self.dtype, self.device,
+            state_manager=self.state_manager)
         builder.add_batch(batch)
         max_pos = getattr(sh, "max_position_embeddings", None)
         if max_pos is not None and builder.position_ids and max(builder.position_ids) >= max_pos:
@@ -318,7 +320,11 @@ class BatchFillExecutor:
                                 f"(max_position_embeddings = {max_pos})")
         inputs = builder.build_language_model_parameters()
         params = LanguageModelParameters(inputs.attention_params, inputs.all_sequences_decode,
-                                         inputs.selected_token_ids_tensor, inputs.image_row_index)
+                                         inputs.selected_token_ids_tensor, inputs.image_row_index,
+                                         sequence_state=inputs.sequence_state)
+        if inputs.logit_rows:
+            self._execute_with_logits(batch, inputs, params)
+            return
         if not inputs.selected_token_ids:
             # nothing samples: the forward still has to run for its cache writes
             self.language_model.language_model.forward_hidden(
@@ -333,6 +339,30 @@ class BatchFillExecutor:
         sampled = sampled.tolist()                      # the step's only device sync
 
         self._deliver(batch, sampled)
+
+
+    def _execute_with_logits(self, batch: BatchRequest, inputs, params: LanguageModelParameters) -> None:
+        """A step in which some request asked for the logits of given rows (Fill.logit_rows): the model's output head runs
+        on those rows and on the sampling rows together; each request's processors get their rows' logits, the sampling
+        rows are sampled from the same logits (greedy, like the model's own forward)."""
+        want = inputs.logit_rows + list(inputs.selected_token_ids)
+        params.selected_token_ids = torch.tensor(want, dtype=torch.int64).to(self.device)
+        lm = self.language_model
+        logits = lm.forward_logits(inputs.input_ids, inputs.image_features, inputs.position_ids, params)
+        if logits.shape[0] != len(want):             # (an all-decode batch of a model that returns every row)
+            logits = logits[params.selected_token_ids]
+        at = 0
+        for rcb, inst in batch:
+            n = len(inst.logit_rows) if isinstance(inst, Fill) and inst.logit_rows else 0
+            if n:
+                for p in rcb.output_token_processors:
+                    p.append_logits(logits[at:at + n], inst)
+                at += n
+        n_logit = len(inputs.logit_rows)
+        if inputs.selected_token_ids:
+            self._deliver(batch, torch.argmax(logits[n_logit:], dim=-1).tolist())
+        else:
+            batch.step()
 
 
 class BatchImageEmbedExecutor:

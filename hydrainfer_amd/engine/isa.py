@@ -36,9 +36,15 @@ class Fill(Instruction):
         self.sample_dst = sample_dst
         self.hashes = hashes
         self.is_chunked = False   # a chunk's sampled token is discarded (executor.py:163-165)
+        # extension: indices into token_ids whose logits the request's output processors are handed
+        # (OutputTokenProcessor.append_logits) — scoring a given text instead of sampling
+        self.logit_rows: Optional[List[int]] = None
 
     def _split_common(self, rest: "Fill", chunk_size: int) -> None:
         self.insert_next(rest)
+        if self.logit_rows is not None:
+            rest.logit_rows = [r - chunk_size for r in self.logit_rows if r >= chunk_size]
+            self.logit_rows = [r for r in self.logit_rows if r < chunk_size]
         self.token_ids = self.token_ids[:chunk_size]
         self.position_ids = self.position_ids[:chunk_size]
         self.cache_ids = self.cache_ids[:chunk_size]
@@ -125,9 +131,28 @@ class PullCache(Instruction):
         return "PR"
 
 
+class AwaitTokens(Instruction):
+    """Extension: the request's text is not complete yet — its client hands it over in pieces (a streamed prompt, a
+    replayed trace).  The request keeps its cache blocks and state slot and sits out every step until an instruction has
+    been linked in behind this one (`extend`), or the client says that nothing more comes (`closed`)."""
+    closed = False
+
+    def ready(self) -> bool:
+        return self.closed or not isinstance(self.next, EmptyInstruction) or self.next.next is not None
+
+    def __repr__(self):
+        return "AW"
+
+
 class InstructionList:
     def __init__(self, head: Instruction, tail: Instruction, curr: Instruction):
         self.head, self.tail, self.curr = head, tail, curr
+
+    def extend(self, inst: Instruction) -> None:
+        """Link an instruction in at the end of a chain that is already running."""
+        self.tail.prev.insert_next(inst)
+        if self.curr is None or self.curr is self.tail:
+            self.curr = inst
 
     def __iter__(self):
         node = self.head

@@ -347,6 +347,10 @@ class EPDNode:
             self.kv_cache_block_manager.realloc(rcb.virtual_kv_cache, 0)
         if rcb.virtual_image_cache is not None and self.image_cache_block_manager is not None:
             self.image_cache_block_manager.realloc(rcb.virtual_image_cache, 0)
+        sm = self.batch_scheduler.context.state_manager
+        if sm is not None and rcb.state_slot is not None:
+            sm.free(rcb.state_slot)
+            rcb.state_slot = None
 
 
 class LocalCluster:

@@ -30,12 +30,18 @@ class FillInputs:
     selected_token_ids: List[int]
     selected_token_ids_tensor: Optional[Tensor]   # int64 on the device
     image_row_index: Optional[Tensor] = None      # int64 on the device: rows that are image tokens
+    sequence_state: Optional[object] = None       # SequenceState of the batch (models with per-sequence state rows)
+    logit_rows: Optional[List[int]] = None        # rows of the batch whose logits a request asked for (Fill.logit_rows)
 
 
 class LanguageModelParametersBuilder:
     def __init__(self, image_block_manager, kv_cache_block_manager, n_layers: int, n_qo_heads: int,
                  n_kv_heads: int, head_dim: int, image_token_id: int, dtype: torch.dtype,
-                 device: torch.device):
+                 device: torch.device, state_manager=None):
+        self.state_manager = state_manager        # memory.state_slots.StateSlotManager or None
+        self.state_slots: List[int] = []
+        self.token_seq: List[int] = []
+        self.logit_rows: List[int] = []
         self.image_block_manager = image_block_manager
         self.kv_cache_block_manager = kv_cache_block_manager
         self.n_layers, self.n_qo_heads, self.head_dim = n_layers, n_qo_heads, head_dim
@@ -54,6 +60,12 @@ class LanguageModelParametersBuilder:
         if isinstance(inst, ImageEmbedFill):
             self.image_slot_ids += self.image_block_manager.v2p(rcb.virtual_image_cache,
                                                                 inst.image_token_cache_ids)
+        if inst.logit_rows:
+            self.logit_rows += [len(self.token_ids) + r for r in inst.logit_rows]
+        if self.state_manager is not None:
+            assert rcb.state_slot is not None, "the scheduler gives every request of a stateful model a state slot"
+            self.token_seq += [len(self.state_slots)] * len(inst.token_ids)
+            self.state_slots.append(rcb.state_slot)
         self.token_ids += inst.token_ids
         self.position_ids += inst.position_ids
         if inst.sample:
@@ -80,7 +92,7 @@ class LanguageModelParametersBuilder:
         assert n_image_rows == n_img, "image token rows and cached image embeddings differ"
         image_rows = [i for i, t in enumerate(self.token_ids) if t == self.image_token_id] if n_img else []
         flat = self._to_device(self.token_ids + self.position_ids + self.selected_token_ids +
-                               self.image_slot_ids + image_rows)
+                               self.image_slot_ids + image_rows + self.state_slots + self.token_seq)
         input_ids, position_ids = flat[:n], flat[n:2 * n]
         selected = flat[2 * n:2 * n + n_sel].to(torch.int64) if n_sel else None
         image_features = None
@@ -92,6 +104,12 @@ class LanguageModelParametersBuilder:
             self.attention_params_builder.add_kv_cache(
                 KVCache.from_token_cache(self.kv_cache_block_manager.get_layer_cache(layer_id)))
         attn = self.attention_params_builder.build_attention_parameters()
-        row_index = flat[2 * n + n_sel + n_img:].to(torch.int64) if n_img else None
+        row_index = flat[2 * n + n_sel + n_img:2 * n + n_sel + 2 * n_img].to(torch.int64) if n_img else None
+        seq_state = None
+        if self.state_manager is not None:
+            from hydrainfer_amd._C.kernel.stream_ops import SequenceState
+            off = 2 * n + n_sel + 2 * n_img
+            n_seq = len(self.state_slots)
+            seq_state = SequenceState(self.state_manager.state, flat[off:off + n_seq], flat[off + n_seq:off + n_seq + n])
         return FillInputs(input_ids, position_ids, image_features, attn, attn[0].all_sequences_decode,
-                          self.selected_token_ids, selected, row_index)
+                          self.selected_token_ids, selected, row_index, seq_state, self.logit_rows or None)

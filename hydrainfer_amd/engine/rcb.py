@@ -60,6 +60,10 @@ class OutputTokenProcessor:
     def append_token_id(self, token_id: int, is_last_token: bool = False) -> None:
         raise NotImplementedError
 
+    def append_logits(self, logits, instruction) -> None:
+        """Extension: the logits [n, vocab] (a float tensor on the model's device) of the rows `instruction.logit_rows`
+        asked for.  Ignored unless a processor wants them."""
+
     def fail(self, exc: BaseException) -> None:
         """The request was terminated by the engine (a migration that failed twice, a node that died): the reference
         pushes a None token to the stream (hydrainfer/cluster/epdnode.py:440-442, `(request_id, None)`)."""
@@ -83,6 +87,7 @@ class RequestControlBlock:
         self.virtual_kv_cache: Optional[VirtualTokenCache] = None
         self.virtual_image_cache: Optional[VirtualTokenCache] = None
         self.sid: int = -1
+        self.state_slot: Optional[int] = None     # models with per-sequence state rows: the slot this request owns (memory/state_slots.py)
         self.output_token_processors: List[OutputTokenProcessor] = []
         self.output_token_ids: List[int] = []
         self.scenario_type: Optional[ScenarioType] = None

@@ -16,7 +16,7 @@ from collections import deque
 from dataclasses import dataclass
 from typing import Deque, List, Optional
 
-from hydrainfer_amd.engine.isa import Fill, ImageEmbed, ImageEmbedFill, PullCache, TextFill
+from hydrainfer_amd.engine.isa import AwaitTokens, Fill, ImageEmbed, ImageEmbedFill, PullCache, TextFill
 from hydrainfer_amd.engine.rcb import BatchRequest, RequestControlBlock
 from hydrainfer_amd.memory.token_cache_manger import BlockTableManager
 
@@ -41,6 +41,7 @@ class BatchSchedulerConfig:
 class BatchSchedulerContext:
     kv_cache_block_manager: Optional[BlockTableManager]
     image_cache_block_manager: Optional[BlockTableManager]
+    state_manager: Optional[object] = None      # memory.state_slots.StateSlotManager: models with per-sequence state rows
 
 
 class BatchScheduler:
@@ -129,6 +130,13 @@ class BatchScheduler:
         for rcb in self.running:
             inst = rcb.current_instruction()
             if isinstance(inst, Fill):
+                if self.context.state_manager is not None and rcb.state_slot is None:
+                    # a request of a stateful model owns one state slot from its first fill to its end
+                    slot = self.context.state_manager.allocate()
+                    if slot < 0:
+                        deferred.add(id(rcb))
+                        continue
+                    rcb.state_slot = slot
                 vc = rcb.virtual_kv_cache
                 if vc is not None and len(inst.cache_ids) == 1:
                     # a decode step (one token): 15 times of 16 its slot lies inside the last block already
@@ -181,6 +189,9 @@ class BatchScheduler:
         self.running_cnt = len(self.running)
         if not self.running:
             return BatchRequest()
+        for rcb in self.running:           # requests whose next piece of text has arrived (or will never come) move on
+            while isinstance(rcb.current_instruction(), AwaitTokens) and rcb.current_instruction().ready():
+                rcb.step()
         deferred = self._grow_caches()
 
         embeds, prefills, decodes = [], [], []
@@ -188,8 +199,8 @@ class BatchScheduler:
         next_step: List[RequestControlBlock] = []
         for rcb in self.running:
             inst = rcb.current_instruction()
-            if id(rcb) in deferred:
-                next_step.append(rcb)      # no room in the pool this step
+            if id(rcb) in deferred or isinstance(inst, AwaitTokens):
+                next_step.append(rcb)      # no room in the pool this step / waiting for its client's next tokens
             elif isinstance(inst, Fill):
                 (decodes if len(inst.token_ids) == 1 else prefills).append(rcb)
             elif isinstance(inst, ImageEmbed):

@@ -38,13 +38,24 @@ def build_node(name: str, node_type: str, language_model, vision_model, lm_shape
                                                      keep_row_major=not release_prefill_weights)
     # one node of MI355Xs: every rank is a same-host peer, so pulls take the IPC path
     ctx = TokenCacheBlockManagerContext(rank=rank, rank2host={r: "localhost" for r in range(max(world_size, rank + 1))})
-    kv = img = None
+    kv = img = state = None
+    inner = getattr(language_model, "language_model", None)
     if nt.has_kv_cache:
+        # what a token leaves in the cache is the model's business: K and V of every KV head (the default), or whatever
+        # its cache_spec names (one latent row per token and layer run)
+        spec = {"n_layers": lm_shape.num_hidden_layers, "n_tokens": 2, "n_heads": lm_shape.num_key_value_heads,
+                "head_size": lm_shape.head_dim}
+        if hasattr(inner, "cache_spec"):
+            spec = inner.cache_spec()
         kv = TokenCacheBlockManager(TokenCacheBlockManagerConfig(
-            n_layers=lm_shape.num_hidden_layers, n_tokens=2, n_blocks=kv_blocks, block_size=16,
-            n_heads=lm_shape.num_key_value_heads, head_size=lm_shape.head_dim, dtype=_DTYPE_NAMES[dtype],
-            device=str(device)), ctx)
-    if nt.has_image_cache:
+            n_blocks=kv_blocks, block_size=16, dtype=_DTYPE_NAMES[dtype], device=str(device),
+            shareable=vision_model is not None or world_size > 1 or node_type != "EPD", **spec), ctx)
+        sspec = inner.state_spec() if hasattr(inner, "state_spec") else None
+        if sspec is not None:
+            # rows a sequence carries from step to step: one slot per request that can be live at once
+            from hydrainfer_amd.memory.state_slots import StateSlotManager
+            state = StateSlotManager(sched.max_running_requests, sspec["rows"], sspec["width"], device)
+    if nt.has_image_cache and vision_model is not None:
         img = TokenCacheBlockManager(TokenCacheBlockManagerConfig(
             n_layers=1, n_tokens=1, n_blocks=image_blocks, block_size=n_image_tokens,
             n_heads=lm_shape.num_attention_heads, head_size=lm_shape.head_dim, dtype=_DTYPE_NAMES[dtype],
@@ -52,14 +63,14 @@ def build_node(name: str, node_type: str, language_model, vision_model, lm_shape
     fill = None
     if nt.has_language_model:
         decoder = None
-        if graph_decode and nt.enable_decode:
+        if graph_decode and nt.enable_decode and getattr(inner, "supports_graph_decode", True):
             from hydrainfer_amd.engine.graph_decode import GraphedDecoder
             decoder = GraphedDecoder(language_model, kv, max_batch=sched.max_running_requests,
                                      max_blocks_per_seq=max_blocks_per_seq)
-        fill = BatchFillExecutor(language_model, kv, img, dtype, device, graph_decoder=decoder)
+        fill = BatchFillExecutor(language_model, kv, img, dtype, device, graph_decoder=decoder, state_manager=state)
     emb = BatchImageEmbedExecutor(vision_model, img, lm_shape.num_attention_heads, lm_shape.head_dim, dtype,
-                                  device, use_graphs=graph_decode) if nt.has_vision_model else None
-    scheduler = BatchScheduler(sched, BatchSchedulerContext(kv, img))
+                                  device, use_graphs=graph_decode) if nt.has_vision_model and vision_model is not None else None
+    scheduler = BatchScheduler(sched, BatchSchedulerContext(kv, img, state))
     return EPDNode(name, nt, scheduler, InstructionExecutor(fill, emb), kv, img, eager_migrate=eager_migrate)
 
 

@@ -26,5 +26,8 @@ class KVCache:
     @classmethod
     def from_token_cache(cls, token_cache: TokenCache) -> "KVCache":
         tensors = token_cache.get_caches()
+        if len(tensors) == 1:
+            # a latent cache: keys and values are both read from the one row a token leaves
+            return cls(tensors[0], tensors[0])
         assert len(tensors) == 2
         return cls(tensors[0], tensors[1])

@@ -41,6 +41,9 @@ class TokenCacheBlockManagerConfig:
     head_size: int = 128
     dtype: str = "fp16"  # 'bf16' accepted (extension; reference str2dtype knows fp16/fp32 only)
     device: str = "cuda:0"
+    shareable: bool = True   # False: a pool no other process ever maps (a collocated node of a text-only model) — no IPC
+                             # handle, no migration backend
+    fill: str = "randn"
 
 
 @dataclass
@@ -132,7 +135,11 @@ class TokenCacheBlockManager(BlockTableManager):
         # that K and V of one token do not share an HBM channel (memory/kv_pool.py)
         self.cache_tensor = kv_pool.allocate_kv_pool(
             (self.n_layers, self.n_tokens, n_blocks, config.block_size, self.n_heads, self.head_size),
-            self.dtype, self.device, fill="randn")
+            self.dtype, self.device, fill=config.fill)
+        if not config.shareable:
+            super().__init__(n_blocks, config.block_size, context.rank, [])
+            self.migrate_stream = self.migrate_manager = None
+            return
         super().__init__(n_blocks, config.block_size, context.rank, get_ipc_mem_handle(self.cache_tensor))
         self.migrate_stream = torch.cuda.Stream(device=self.device)
         self.migrate_manager = CommunicationBackendManager(
@@ -146,13 +153,16 @@ class TokenCacheBlockManager(BlockTableManager):
 
     def migrate_blocks(self, src_virtual_cache: VirtualTokenCache,
                        dst_virtual_cache: VirtualTokenCache, is_send: bool = False) -> None:
+        if self.migrate_manager is None:
+            raise RuntimeError("this cache pool was built with shareable=False: its blocks cannot be migrated")
         self.migrate_manager.migrate_blocks(src_virtual_cache, dst_virtual_cache, is_send)
 
     def needs_sender(self, src_virtual_cache: VirtualTokenCache, dst_virtual_cache: VirtualTokenCache) -> bool:
         return self.migrate_manager.needs_sender(src_virtual_cache.rank, dst_virtual_cache.rank)
 
     def synchronize(self) -> None:
-        self.migrate_stream.synchronize()
+        if self.migrate_stream is not None:
+            self.migrate_stream.synchronize()
 
     @classmethod
     def compute_n_blocks(cls, config: TokenCacheBlockManagerConfig, memory: int) -> int:

@@ -57,6 +57,8 @@ class LanguageModelParameters:
                                                  # spares the nonzero() sync of a boolean-mask assignment)
     step_head: Optional[StepHead] = None         # decode loops: metadata advance / look-ahead feed folded into the step's
                                                  # first launch (hx_decode_step_head); the model runs it or raises
+    sequence_state: Optional[object] = None      # models that carry rows from step to step (a token shift): the batch's
+                                                 # sequences and their state slots (_C.kernel.stream_ops.SequenceState)
 
 
 def build_cos_sin(shape: LlamaShape, dtype: torch.dtype, device) -> Tensor:

@@ -36,3 +36,29 @@ class LlavaLanguageModel:
         return torch.argmax(self.forward_logits(input_ids, image_features, position_ids, model_params), dim=-1)
 
     __call__ = forward
+
+
+class TextLanguageModel:
+    """The engine's language-model interface (LlavaLanguageModel's) around a text-only decoder: no image token, no image
+    features.  `language_model` is any model with forward_hidden / forward_logits / forward over (token ids, position
+    ids, LanguageModelParameters) — LlamaForCausalLM, TetepelForCausalLM."""
+
+    def __init__(self, language_model):
+        self.language_model = language_model
+        self.image_token_id = -1                  # no token id is an image placeholder
+
+    def embed(self, input_ids: Tensor, image_features: Optional[Tensor] = None,
+              image_row_index: Optional[Tensor] = None) -> Tensor:
+        if image_features is not None:
+            raise ValueError("a text-only model was handed image features")
+        return self.language_model.embed(input_ids)
+
+    def forward_logits(self, input_ids: Tensor, image_features: Optional[Tensor], position_ids: Tensor,
+                       model_params: LanguageModelParameters) -> Tensor:
+        return self.language_model.forward_logits(self.embed(input_ids, image_features), position_ids, model_params)
+
+    def forward(self, input_ids: Tensor, image_features: Optional[Tensor], position_ids: Tensor,
+                model_params: LanguageModelParameters) -> Tensor:
+        return self.language_model.forward(self.embed(input_ids, image_features), position_ids, model_params)
+
+    __call__ = forward
