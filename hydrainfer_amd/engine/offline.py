@@ -40,10 +40,17 @@ class OfflineInferenceEngine:
                  max_context: int = 4096, kv_cache_gib: Optional[float] = None, warm_up: bool = True):
         self.device = torch.device(device)
         torch.cuda.set_device(self.device)
-        shape = language_model.language_model.shape
-        self.n_image_tokens = (vision_model.shape.image_size // vision_model.shape.patch_size) ** 2
+        inner = language_model.language_model
+        shape = inner.shape
+        # vision_model None: a text-only model (model.llava.TextLanguageModel)
+        self.n_image_tokens = (vision_model.shape.image_size // vision_model.shape.patch_size) ** 2 if vision_model is not None else 0
+        cache_spec = inner.cache_spec() if hasattr(inner, "cache_spec") else None
+        stateful = hasattr(inner, "state_spec") and inner.state_spec() is not None
         blocks_per_seq = (max_context + 15) // 16
         per_block = shape.num_hidden_layers * 2 * 16 * shape.num_key_value_heads * shape.head_dim * 2
+        if cache_spec is not None:
+            per_block = (cache_spec["n_layers"] * cache_spec["n_tokens"] * 16 * cache_spec["n_heads"] * cache_spec["head_size"]
+                         * torch.empty((), dtype=dtype).element_size())
         n_blocks = int(kv_cache_gib * (1 << 30) // per_block) if kv_cache_gib else blocks_per_seq * (max_running_requests + 2)
         sched = BatchSchedulerConfig(priority="prefill", max_running_requests=max_running_requests,
                                      chunked_prefill=True, token_budgets=token_budgets, image_budgets=image_budgets)
@@ -53,9 +60,10 @@ class OfflineInferenceEngine:
         self.cluster = LocalCluster([self.node])
         self.creator = InstructionCreator(image_token_id=language_model.image_token_id,
                                           n_image_tokens_per_image=self.n_image_tokens, block_size=16, ignore_eos=True,
-                                          max_position_embeddings=shape.max_position_embeddings)
-        self.processor = ClipImageProcessor(size=vision_model.shape.image_size)
-        if warm_up:
+                                          max_position_embeddings=shape.max_position_embeddings,
+                                          prefix_cache=not stateful)
+        self.processor = ClipImageProcessor(size=vision_model.shape.image_size) if vision_model is not None else None
+        if warm_up and vision_model is not None:
             warm_library_gemms(language_model, token_budgets, max_running_requests)
             size = vision_model.shape.image_size
             self.node.executor.image_embed_executor.warmup(torch.zeros(1, 3, size, size), image_budgets)
@@ -63,8 +71,8 @@ class OfflineInferenceEngine:
 
     @classmethod
     def from_checkpoint(cls, model_path: str, dtype: torch.dtype = torch.float16, device: str = "cuda:0", **kw):
-        from hydrainfer_amd.model.loader import load_llava
-        lm, vm = load_llava(model_path, dtype, device)
+        from hydrainfer_amd.model.registry import load_model
+        lm, vm = load_model(model_path, dtype, device)       # the model class is chosen by config.json
         return cls(lm, vm, dtype, device, **kw)
 
     def generate(self, requests: List[OfflineRequest]) -> List[OfflineInferenceOutput]:
@@ -72,6 +80,8 @@ class OfflineInferenceEngine:
         rcbs = []
         with quiet_gc():
             for i, r in enumerate(requests):
+                if r.image is not None and self.processor is None:
+                    raise ValueError("this engine serves a text-only model: request with an image")
                 pixels = self.processor.process(r.image) if r.image is not None else None
                 req = TokenRequest(request_id=i, token_ids=list(r.token_ids), pixel_values=pixels,
                                    image_size=(r.image.size[1], r.image.size[0]) if r.image is not None else (0, 0),

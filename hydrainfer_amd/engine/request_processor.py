@@ -25,8 +25,11 @@ class TokenRequest:
 class InstructionCreator:
     def __init__(self, image_token_id: int = 32000, n_image_tokens_per_image: int = 576,
                  block_size: int = 16, ignore_eos: bool = True, eos_token_id: int = 2,
-                 max_position_embeddings: int = 4096):
-        self.max_position_embeddings = max_position_embeddings
+                 max_position_embeddings: int = 4096, prefix_cache: bool = True):
+        self.max_position_embeddings = max_position_embeddings      # None: the model has no positional table
+        # False for models that carry state rows beside the cache: a cached block says nothing about them, so no prompt
+        # is matched against earlier ones
+        self.prefix_cache = prefix_cache
         self.image_token_id = image_token_id
         self.n_image_tokens_per_image = n_image_tokens_per_image
         self.block_size = block_size
@@ -64,7 +67,10 @@ class InstructionCreator:
         n_prompt = len(token_ids)
         # position ids run to n_prompt + max_tokens - 2; the rotary table (cos_sin) has
         # max_position_embeddings rows and the kernels index it unchecked
-        if n_prompt + rcb.sampling_params.max_tokens - 1 > self.max_position_embeddings:
+        if not self.prefix_cache:
+            hashes = None
+        if self.max_position_embeddings is not None and \
+                n_prompt + rcb.sampling_params.max_tokens - 1 > self.max_position_embeddings:
             raise ValueError(f"request {request.request_id}: {n_prompt} prompt tokens + "
                              f"{rcb.sampling_params.max_tokens} generated exceed max_position_embeddings "
                              f"= {self.max_position_embeddings}")

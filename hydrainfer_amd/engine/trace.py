@@ -90,7 +90,7 @@ class TraceReplayer:
         for (rcb, wait), e in zip(parked, entries):
             if rcb.current_instruction() is not wait:
                 raise RuntimeError(f"request {e['id']} did not run in its step (cache pool or state slots exhausted: "
-                                   f"{self.node.kv_cache_block_manager.get_num_avaiable_blocks()} blocks free)")
+                                   f"{len(self.node.kv_cache_block_manager.shared_cache.to_be_evicted)} blocks free)")
         rows = [r for rcb, _ in parked for r in rcb.output_token_processors[0].take()]
         done = [rid for rid in end if rid in self.live]
         for rid in done:

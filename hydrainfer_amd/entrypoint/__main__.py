@@ -12,7 +12,9 @@ import torch
 def main():
     ap = argparse.ArgumentParser(prog="python -m hydrainfer_amd.entrypoint")
     ap.add_argument("--model", default="7b", choices=["7b", "13b", "tiny"])
-    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"])
+    ap.add_argument("--checkpoint", default=None, help="checkpoint directory (config.json + *.safetensors): the model class is "
+                    "chosen by config.json (model.registry) and --model is ignored")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16", "fp32"])
     ap.add_argument("--host", default="127.0.0.1")
     ap.add_argument("--port", type=int, default=8888)
     ap.add_argument("--max-running", type=int, default=64)
@@ -32,10 +34,13 @@ def main():
     from hydrainfer_amd.model.llava import LlavaLanguageModel
     from hydrainfer_amd.model.processor import ClipImageProcessor
     import dataclasses
-    _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    dt = torch.bfloat16 if a.dtype == "bf16" else torch.float16
+    dt = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32}[a.dtype]
+    if a.checkpoint:
+        serve_checkpoint(a, dt, dev)
+        return
+    _lib.lib()
     shape = {"7b": LLAVA_1_5_7B, "13b": LLAVA_1_5_13B, "tiny": LlamaShape(256, 512, 2, 2, 2, 128, 32064)}[a.model]
     cshape = (dataclasses.replace(CLIP_VIT_L_14_336, projector_hidden_size=shape.hidden_size) if a.model != "tiny" else
               ClipShape(hidden_size=128, intermediate_size=256, num_hidden_layers=3, num_attention_heads=2, image_size=336,
@@ -56,6 +61,33 @@ def main():
     tok = HFTokenizer(a.tokenizer) if a.tokenizer else SyntheticTokenizer(image_token_id=itid)
     front = EngineFrontend(LocalCluster([node]), creator, device=dev)
     print(f"serving {a.model} ({a.dtype}, random weights) on http://{a.host}:{a.port}/v1/chat/completions", flush=True)
+    ApiServer(front, tok, ClipImageProcessor(), host=a.host, port=a.port).run()
+
+
+def serve_checkpoint(a, dt, dev):
+    """One collocated replica of the model in a checkpoint directory, whatever registered architecture it is."""
+    from hydrainfer_amd.engine.node import LocalCluster
+    from hydrainfer_amd.engine.request_processor import InstructionCreator
+    from hydrainfer_amd.engine.scheduler import BatchSchedulerConfig
+    from hydrainfer_amd.engine.serve import build_node
+    from hydrainfer_amd.entrypoint import ApiServer, EngineFrontend, HFTokenizer, SyntheticTokenizer
+    from hydrainfer_amd.model.processor import ClipImageProcessor
+    from hydrainfer_amd.model.registry import load_model
+    lm, vision = load_model(a.checkpoint, dt, dev)
+    inner = lm.language_model
+    shape = inner.shape
+    stateful = hasattr(inner, "state_spec") and inner.state_spec() is not None
+    n_img = (vision.shape.image_size // vision.shape.patch_size) ** 2 if vision is not None else 0
+    sched = BatchSchedulerConfig(priority="prefill", max_running_requests=a.max_running, chunked_prefill=True,
+                                 token_budgets=4096, image_budgets=8)
+    per_req = (a.max_tokens + 15) // 16 + 1
+    node = build_node("EPD0", "EPD", lm, vision, shape, dt, dev, kv_blocks=a.max_running * per_req + 64,
+                      image_blocks=2 * a.max_running, n_image_tokens=n_img, sched=sched, max_blocks_per_seq=per_req)
+    creator = InstructionCreator(image_token_id=lm.image_token_id, n_image_tokens_per_image=n_img, block_size=16,
+                                 max_position_embeddings=shape.max_position_embeddings, prefix_cache=not stateful)
+    tok = HFTokenizer(a.tokenizer) if a.tokenizer else SyntheticTokenizer(image_token_id=lm.image_token_id)
+    front = EngineFrontend(LocalCluster([node]), creator, device=dev)
+    print(f"serving {a.checkpoint} ({a.dtype}) on http://{a.host}:{a.port}/v1/chat/completions", flush=True)
     ApiServer(front, tok, ClipImageProcessor(), host=a.host, port=a.port).run()
 
 

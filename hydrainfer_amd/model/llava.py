@@ -45,7 +45,7 @@ class TextLanguageModel:
 
     def __init__(self, language_model):
         self.language_model = language_model
-        self.image_token_id = -1                  # no token id is an image placeholder
+        self.image_token_id = -(1 << 40)          # no token id (nor the -1 of a token still to be sampled) is an image placeholder
 
     def embed(self, input_ids: Tensor, image_features: Optional[Tensor] = None,
               image_row_index: Optional[Tensor] = None) -> Tensor:

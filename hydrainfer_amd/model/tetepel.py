@@ -322,10 +322,17 @@ class TetepelForCausalLM:
         if input_ids.dtype not in (torch.int32, torch.int64):
             raise ValueError("Tetepel takes token ids (its embedding is scaled and copied into the streams)")
         seq = model_params.sequence_state
-        if seq is None:
-            raise ValueError("Tetepel needs LanguageModelParameters.sequence_state (the batch's sequences and their state slots)")
         if position_ids.dtype != torch.int32:
             position_ids = position_ids.to(torch.int32)
+        if seq is None:
+            if self.state_spec() is not None:
+                raise ValueError("Tetepel with a token shift needs LanguageModelParameters.sequence_state (the batch's "
+                                 "sequences and their state slots)")
+            # no state rows: the sequence of every token follows from the batch's portion lengths (no host round trip)
+            q_cu = model_params.attention_params[0].q_cu_seq_lens
+            tok_seq = torch.repeat_interleave(torch.arange(q_cu.numel() - 1, device=q_cu.device), q_cu.diff().long(),
+                                              output_size=input_ids.shape[0]).to(torch.int32)
+            seq = SequenceState(None, None, tok_seq)
         x = stream_embed(input_ids.contiguous(), self.embed_table, sh.embedding_scale, sh.streams)
         for run, li in enumerate(sh.run_order):
             self._mixer(run, li, x, position_ids, model_params.attention_params[run], seq)
