@@ -232,6 +232,7 @@ class hxm_latent_attn_args(ctypes.Structure):
 _MIX_SIGNATURES = {
     "hxm_abi_version": (c_int, []),
     "hxm_last_hip_error": (c_int, []),
+    "hxm_set_option": (c_int, [c_char_p, c_int]),
     "hxm_stream_embed": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_float, c_int64, c_int32, c_int64, c_int64, c_int, c_void_p]),
     "hxm_stream_norm": (c_int, [c_void_p, c_void_p, c_void_p, c_int32, c_float, c_void_p, c_int64, c_int32, c_int64, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),

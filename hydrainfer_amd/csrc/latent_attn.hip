@@ -3,11 +3,12 @@
 // the value map applied afterwards (o = W_uv sum_j p_j c_j) the kernel is multi-query attention whose keys and values
 // are the same rows: score = q~ . c_j * scale, out = sum_j softmax(score)_j c_j.  Scores, weights and sums are float.
 // Sliding window: a query at position i sees keys j with 0 <= i - j < window.
-#include "hx_common.h"
+#include "attn_common.h"
 #include "../../include/hydra_mix.h"
 
 namespace hxm {
 int check_launch();
+int& tile_form();      // 0: row form only (A/B measurements), 1: tile form where it applies
 }
 
 namespace {
@@ -81,6 +82,9 @@ __global__ __launch_bounds__(256) void latent_attn_rows_kernel(hxm_latent_attn_a
   const int32_t lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int32_t* table = a.block_table + a.cu_block_lens[b];
   const typename A::storage* cache = (const typename A::storage*)a.cache;
+  constexpr int kVec = 16 / sizeof(typename A::storage);
+  const bool vec = R % kVec == 0 && a.cache_row_stride % kVec == 0 && a.cache_block_stride % kVec == 0 &&
+                   (reinterpret_cast<uintptr_t>(a.cache) & 15u) == 0;
   float m = -INFINITY, l = 0.f;
   float acc[kMaxCols];
 #pragma unroll
@@ -94,7 +98,17 @@ __global__ __launch_bounds__(256) void latent_attn_rows_kernel(hxm_latent_attn_a
       off = (int64_t)table[j / a.block_size] * a.cache_block_stride + (int64_t)(j % a.block_size) * a.cache_row_stride;
       const typename A::storage* c = cache + off;
       float d = 0.f;
-      for (int i = 0; i < R; ++i) d += q[i] * A::to_float(c[i]);
+      if (vec) {      // 16-byte loads of the row
+        constexpr int N = 16 / sizeof(typename A::storage);
+        typedef typename A::storage VecT __attribute__((ext_vector_type(N)));
+        for (int i = 0; i < R; i += N) {
+          const VecT v = *reinterpret_cast<const VecT*>(c + i);
+#pragma unroll
+          for (int e = 0; e < N; ++e) d += q[i + e] * A::to_float(v[e]);
+        }
+      } else {
+        for (int i = 0; i < R; ++i) d += q[i] * A::to_float(c[i]);
+      }
       s = d;
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -127,6 +141,204 @@ __global__ __launch_bounds__(256) void latent_attn_rows_kernel(hxm_latent_attn_a
     const int i = lane + 64 * k;
     if (i < R && live) og[i] = A::from_float(acc[k] * g);
   }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Tile form (bfloat16): one wave per 16 rows, a row being a (token, head) pair of ONE sequence's portion, heads fastest —
+// sixteen heads of a decoded token, or a few tokens times a few heads.  All rows of a tile read the same keys, which go
+// by in chunks of 32: S = Q C^T and O += P C are 16x16x32 MFMAs.  The chunk's rows come straight from the paged cache
+// into the B operands of S (a lane's 16 bytes are 8 consecutive columns of one key's row); for O the same registers are
+// written to the wave's LDS transposed (CT[column][key], two keys a word), P goes through LDS from the accumulator
+// layout to the A layout.  Inside a chunk the 32 keys are summed in the order slot = 2 * (key % 16) + key / 16 in both
+// operands, so that a lane's two keys are neighbours.  No barriers: a wave shares nothing with its neighbours.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kCtStride = 36;      // u16 per CT / P row: 32 slots + 4 (72 bytes: the four 16-lane groups of a write hit different banks)
+
+template <int KK>                  // ceil(kv_rank / 32), 1 .. 16
+__global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_args a, int tiles_per_seq, int waves_per_block) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (wave >= waves_per_block) return;
+  const int64_t item = (int64_t)blockIdx.x * waves_per_block + wave;
+  if (item >= (int64_t)a.n_seq * tiles_per_seq) return;
+  const int b = (int)(item / tiles_per_seq), tile = (int)(item % tiles_per_seq);
+  const int H = a.n_heads, R = a.kv_rank;
+  const int q0 = a.q_cu[b];
+  const int n_rows = (a.q_cu[b + 1] - q0) * H;
+  if (tile * 16 >= n_rows) return;
+  const int g = lane >> 4, c = lane & 15;
+  const int R16 = (R + 15) / 16 * 16;
+  u16* ct = reinterpret_cast<u16*>(lds) + (size_t)wave * (R16 + 16) * kCtStride;
+  u16* pl = ct + (size_t)R16 * kCtStride;
+  const u16* cache = (const u16*)a.cache;
+  const int32_t* table = a.block_table + a.cu_block_lens[b];
+
+  // the queries: lane (g, c) holds row c, columns 32 kk + 8 g .. + 7
+  const int last_row = min(tile * 16 + 15, n_rows - 1);
+  u16x8 qf[KK];
+  {
+    const int r = min(tile * 16 + c, n_rows - 1);
+    const u16* qg = (const u16*)a.q + (int64_t)(q0 + r / H) * a.q_token_stride + (int64_t)(r % H) * a.q_head_stride;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int col = 32 * kk + 8 * g;
+      if (col < R) qf[kk] = *reinterpret_cast<const u16x8*>(qg + col);
+      else qf[kk] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+  // the rows this lane holds of S and O: 4 g + i
+  int pos[4], lo[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 16 + 4 * g + i;
+    if (r < n_rows) {
+      pos[i] = a.positions[q0 + r / H];
+      lo[i] = a.window > 0 ? max(0, pos[i] - a.window + 1) : 0;
+    } else {
+      pos[i] = -1;      // sees nothing
+      lo[i] = 0;
+    }
+  }
+  // the keys any row of the tile sees: lane (., c) looks at row c, the sixteen are reduced by shuffles
+  int k_min, k_max;
+  {
+    const int r = min(tile * 16 + c, last_row);
+    const int pr = a.positions[q0 + r / H];
+    k_max = pr;
+    k_min = a.window > 0 ? max(0, pr - a.window + 1) : 0;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+      k_max = max(k_max, __shfl_xor(k_max, off, 64));
+      k_min = min(k_min, __shfl_xor(k_min, off, 64));
+    }
+  }
+
+  float m[4], l[4];
+  f32x4 acc[KK * 2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { m[i] = -1.0e30f; l[i] = 0.f; }
+#pragma unroll
+  for (int n = 0; n < KK * 2; ++n) acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int key0 = k_min; key0 <= k_max; key0 += 32) {
+    f32x4 sc[2];
+    u16x8 cf[2][KK];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int key = min(key0 + 16 * s + c, k_max);        // (a key past the last one repeats it; masked below)
+      const u16* row = cache + (int64_t)table[key / a.block_size] * a.cache_block_stride +
+                       (int64_t)(key % a.block_size) * a.cache_row_stride;
+      sc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        const int col = 32 * kk + 8 * g;
+        if (col < R) cf[s][kk] = *reinterpret_cast<const u16x8*>(row + col);
+        else cf[s][kk] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        sc[s] = Mfma<BF16>::mma(qf[kk], cf[s][kk], sc[s]);
+      }
+    }
+    // the chunk, transposed, for the second product: CT[column][slot], slot = 2 c + s
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int col = 32 * kk + 8 * g;
+      if (col < R) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          *reinterpret_cast<uint32_t*>(ct + (size_t)(col + j) * kCtStride + 2 * c) =
+              (uint32_t)cf[0][kk][j] | ((uint32_t)cf[1][kk][j] << 16);
+      }
+    }
+    // softmax of the rows 4 g + i over this chunk (sc[s][i] is key key0 + 16 s + c)
+    float p[2][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const int key = key0 + 16 * s + c;
+        const bool seen = key >= lo[i] && key <= pos[i];
+        const float v = seen ? sc[s][i] * a.scale : -INFINITY;
+        p[s][i] = v;
+        mx = fmaxf(mx, v);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
+      const float m_new = fmaxf(m[i], mx);
+      const float corr = __expf(m[i] - m_new);
+      float ps = 0.f;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        p[s][i] = __expf(p[s][i] - m_new);       // exp(-inf) = 0 for a key the row does not see
+        ps += p[s][i];
+      }
+      ps += __shfl_xor(ps, 1, 64);
+      ps += __shfl_xor(ps, 2, 64);
+      ps += __shfl_xor(ps, 4, 64);
+      ps += __shfl_xor(ps, 8, 64);
+      l[i] = l[i] * corr + ps;
+      m[i] = m_new;
+#pragma unroll
+      for (int n = 0; n < KK * 2; ++n) acc[n][i] *= corr;
+      *reinterpret_cast<uint32_t*>(pl + (size_t)(4 * g + i) * kCtStride + 2 * c) =
+          (uint32_t)BF16::from_float(p[0][i]) | ((uint32_t)BF16::from_float(p[1][i]) << 16);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // O += P C: A = P[row c][slots 8 g ..], B = CT[column 16 n + c][slots 8 g ..]
+    u16x8 pf;
+    {
+      const u16x4 x0 = *reinterpret_cast<const u16x4*>(pl + (size_t)c * kCtStride + 8 * g);
+      const u16x4 x1 = *reinterpret_cast<const u16x4*>(pl + (size_t)c * kCtStride + 8 * g + 4);
+      pf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+    }
+#pragma unroll
+    for (int n = 0; n < KK * 2; ++n) {
+      if (16 * n < R) {
+        const u16* src = ct + (size_t)(16 * n + c) * kCtStride + 8 * g;
+        const u16x4 x0 = *reinterpret_cast<const u16x4*>(src);
+        const u16x4 x1 = *reinterpret_cast<const u16x4*>(src + 4);
+        const u16x8 vf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        acc[n] = Mfma<BF16>::mma(pf, vf, acc[n]);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();      // the reads are done before the next chunk is written
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 16 + 4 * g + i;
+    if (r >= n_rows) continue;
+    const int t = q0 + r / H, h = r % H;
+    float gsc = 1.0f / l[i];
+    if (a.gate_pre) {
+      const float z = BF16::to_float(((const u16*)a.gate_pre)[(int64_t)t * a.gate_stride + h]);
+      gsc = gsc / (1.0f + __expf(-z));
+    }
+    u16* og = (u16*)a.out + (int64_t)t * a.out_token_stride + (int64_t)h * a.out_head_stride;
+#pragma unroll
+    for (int n = 0; n < KK * 2; ++n) {
+      const int col = 16 * n + c;
+      if (col < R) og[col] = BF16::from_float(acc[n][i] * gsc);
+    }
+  }
+}
+
+template <int KK>
+int launch_tile(const hxm_latent_attn_args& a, hipStream_t s) {
+  const int R16 = (a.kv_rank + 15) / 16 * 16;
+  const size_t per_wave = (size_t)(R16 + 16) * kCtStride * sizeof(u16);
+  int waves = 4;
+  while (waves > 1 && per_wave * waves > 64 * 1024) waves >>= 1;
+  const int tiles_per_seq = (int)(((int64_t)a.max_q_len * a.n_heads + 15) / 16);
+  const int64_t items = (int64_t)a.n_seq * tiles_per_seq;
+  const dim3 grid((unsigned)((items + waves - 1) / waves));
+  latent_attn_tile_kernel<KK><<<grid, dim3(256), per_wave * waves, s>>>(a, tiles_per_seq, waves);
+  return hxm::check_launch();
 }
 
 }  // namespace
@@ -165,6 +377,21 @@ extern "C" int hxm_latent_attention(const hxm_latent_attn_args* args, void* stre
   if (!a.out || !a.q || !a.cache || !a.tok_seq || !a.positions || !a.q_cu || !a.block_table || !a.cu_block_lens) return HX_ERR_NULL;
   if (a.cache_row_stride < a.kv_rank) return HX_ERR_STRIDE;
   hipStream_t s = (hipStream_t)stream;
+  if (a.max_q_len < 1) return HX_ERR_SHAPE;
+  const bool aligned = a.kv_rank % 8 == 0 && a.cache_row_stride % 8 == 0 && a.cache_block_stride % 8 == 0 &&
+                       a.q_token_stride % 8 == 0 && a.q_head_stride % 8 == 0 && aligned16(a.cache) && aligned16(a.q);
+  if (a.dtype == HX_BF16 && aligned && hxm::tile_form()) {
+    switch ((a.kv_rank + 31) / 32) {
+      case 1: return launch_tile<1>(a, s);
+      case 2: return launch_tile<2>(a, s);
+      case 3: return launch_tile<3>(a, s);
+      case 4: return launch_tile<4>(a, s);
+      case 5: case 6: return launch_tile<6>(a, s);
+      case 7: case 8: return launch_tile<8>(a, s);
+      case 9: case 10: case 11: case 12: return launch_tile<12>(a, s);
+      default: return launch_tile<16>(a, s);
+    }
+  }
   const int64_t items = (int64_t)a.n_tokens * a.n_heads;
   const dim3 grid((unsigned)((items + 3) / 4));
   const size_t lds = (size_t)4 * a.kv_rank * sizeof(float);

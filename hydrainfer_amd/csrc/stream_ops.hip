@@ -19,6 +19,10 @@ int check_launch() {
   }
   return HX_OK;
 }
+int& tile_form() {
+  static int v = 1;
+  return v;
+}
 }  // namespace hxm
 
 namespace {
@@ -170,6 +174,13 @@ int launch_embed(float* x, const void* table, const void* ids, int ids64, float 
 
 extern "C" int hxm_abi_version(void) { return HXM_ABI_VERSION; }
 extern "C" int hxm_last_hip_error(void) { return hxm::last_hip_error(); }
+extern "C" int hxm_set_option(const char* name, int value) {
+  if (name && __builtin_strcmp(name, "attn_tile_form") == 0) {
+    hxm::tile_form() = value ? 1 : 0;
+    return HX_OK;
+  }
+  return HX_ERR_UNSUPPORTED;
+}
 
 extern "C" int hxm_stream_embed(float* x, const void* table, const void* ids, int ids_are_int64, float scale,
                                 int64_t n_tokens, int32_t n_streams, int64_t width, int64_t vocab, int dtype, void* stream) {

@@ -26,6 +26,9 @@ extern "C" {
 
 int hxm_abi_version(void);
 int hxm_last_hip_error(void);
+/* A/B measurements in one process: "attn_tile_form" = 0 keeps bfloat16 attention on the row form (one wave per token
+ * and head) instead of the MFMA tile form.  Results agree within bfloat16 rounding. */
+int hxm_set_option(const char* name, int value);
 
 /* x[t, s, :] = table[ids[t], :] * scale for every stream s.  x: float [n_tokens, n_streams, width]; table: dtype
  * [vocab, width]; ids: int32 or int64.  An id outside [0, vocab) writes zeros. */

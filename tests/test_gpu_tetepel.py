@@ -228,14 +228,23 @@ def test_latent_attention_kernel_window_edges_page_borders_and_far_keys(R, H, wi
         ch = cache.to(dtype)
         qd = q[idx].to(dtype).to(DEV)
         out = latent_attention(qd, ch, tok_seq[idx].to(DEV), positions[idx].to(DEV), q_cu.to(DEV), table, cu_blocks, scale,
-                               window, 4, gate_pre=gate[idx].to(dtype).to(DEV))
+                               window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV))
         _close(out.float().cpu(), ref[idx], tol, f"latent attention {dtype}")
         # strided query / result layouts (heads outermost), as the model hands them over
         qh = qd.transpose(0, 1).contiguous()
         oh = torch.empty_like(qh)
         latent_attention(qh.transpose(0, 1), ch, tok_seq[idx].to(DEV), positions[idx].to(DEV), q_cu.to(DEV), table, cu_blocks,
-                         scale, window, 4, gate_pre=gate[idx].to(dtype).to(DEV), out=oh.transpose(0, 1))
+                         scale, window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV), out=oh.transpose(0, 1))
         assert torch.equal(oh.transpose(0, 1), out)
+        if dtype == torch.bfloat16:      # the row form of the same kernel (what float32 runs on) agrees with the tile form
+            from hydrainfer_amd import _lib
+            _lib.mix_lib().hxm_set_option(b"attn_tile_form", 0)
+            try:
+                rows = latent_attention(qd, ch, tok_seq[idx].to(DEV), positions[idx].to(DEV), q_cu.to(DEV), table, cu_blocks,
+                                        scale, window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV))
+            finally:
+                _lib.mix_lib().hxm_set_option(b"attn_tile_form", 1)
+            _close(rows.float().cpu(), ref[idx], tol, "latent attention, row form in bfloat16")
 
 
 def test_latent_norm_cache_kernel_writes_the_rows_it_is_told_to():
