@@ -79,6 +79,11 @@ def parse():
     p.add_argument("--no-ragged", action="store_true", help="skip whole_step_ragged (the decode step on ragged batches)")
     p.add_argument("--no-null-step", action="store_true",
                    help="skip whole_step.null_step (the launch structure's ceiling: the step with math-free stand-in launches)")
+    p.add_argument("--design", default=None, choices=["tetepel"],
+                   help="instead of the default workload: prefill / decode throughput of this model design at layer sizes of a "
+                        "real model (random weights) beside the Llama decoder at equal size, and its kernels against the Llama "
+                        "path's like kernels as fractions of their rooflines (hydrainfer_amd/utils/design_bench.py); 1 GPU")
+    p.add_argument("--design-sizes", default="w2048,w4096")
     p.add_argument("--dry-run", action="store_true",
                    help="launch plumbing only (ranks, rendezvous, barrier, max-over-ranks timing of empty steps): "
                         "no GPU is touched; the JSON line says dry_run")
@@ -1487,8 +1492,25 @@ def leg_13b_child(args):
     return leg
 
 
+def design_leg(args):
+    """`--design tetepel`: one JSON line — the design's throughput and kernel table beside the Llama decoder's."""
+    from hydrainfer_amd.utils import design_bench
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float16
+    if dtype != torch.bfloat16:
+        raise SystemExit("--design: the design's 16-bit dtype is bf16")
+    res = design_bench.run(dtype, dev, tuple(args.design_sizes.split(",")))
+    first = next(iter(res["throughput"].values()))
+    print(json.dumps({"metric": f"{args.design}_decode_tok_s", "value": first["tetepel"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1,
+                      "higher_is_better": True, "dtype": "bf16", "data": "synthetic", "design": args.design, **res}))
+    return 0
+
+
 def main():
     args = parse()
+    if args.design:
+        return design_leg(args)
     launch_ranks_if_needed(args)             # N > 1 without WORLD_SIZE: this process only starts the ranks
     if args.dry_run:
         return dry_run(args)

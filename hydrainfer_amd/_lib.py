@@ -212,8 +212,8 @@ def lib() -> ctypes.CDLL:
 # ---------------------------------------------------------------------------------------------------------
 MIX_LIB_PATH = os.environ.get("HX_MIX_LIB_PATH") or os.path.join(_HERE, "lib", "libhydra_mix.so")
 HXM_ABI_VERSION = 1
-HXM_MAX_STREAMS = 8
-HXM_MAX_LATENT = 512
+HXM_MAX_STREAMS = 16
+HXM_MAX_LATENT = 1024
 
 
 class hxm_latent_attn_args(ctypes.Structure):

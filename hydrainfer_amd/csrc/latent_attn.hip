@@ -380,7 +380,7 @@ extern "C" int hxm_latent_attention(const hxm_latent_attn_args* args, void* stre
   if (a.max_q_len < 1) return HX_ERR_SHAPE;
   const bool aligned = a.kv_rank % 8 == 0 && a.cache_row_stride % 8 == 0 && a.cache_block_stride % 8 == 0 &&
                        a.q_token_stride % 8 == 0 && a.q_head_stride % 8 == 0 && aligned16(a.cache) && aligned16(a.q);
-  if (a.dtype == HX_BF16 && aligned && hxm::tile_form()) {
+  if (a.dtype == HX_BF16 && aligned && a.kv_rank <= 512 && hxm::tile_form()) {
     switch ((a.kv_rank + 31) / 32) {
       case 1: return launch_tile<1>(a, s);
       case 2: return launch_tile<2>(a, s);

@@ -114,17 +114,17 @@ __global__ __launch_bounds__(256) void stream_norm_kernel(const float* __restric
   }
 }
 
-template <typename A>
+template <typename A, int MS>      // MS: 4 / 8 / 16 >= the number of streams (the loops are unrolled)
 __global__ __launch_bounds__(256) void stream_update_kernel(float* __restrict__ x, const typename A::storage* __restrict__ y,
                                                             int64_t y_stride, const typename A::storage* __restrict__ gate_pre,
                                                             int64_t gate_stride, const float* __restrict__ gate_b,
                                                             const float* __restrict__ mix, const float* __restrict__ out_w,
                                                             int32_t S, int64_t W) {
-  __shared__ float m[HXM_MAX_STREAMS * HXM_MAX_STREAMS + HXM_MAX_STREAMS];
+  __shared__ float m[MS * MS + MS];
   if (threadIdx.x < S * S) m[threadIdx.x] = mix[threadIdx.x];
-  if (threadIdx.x < S) m[HXM_MAX_STREAMS * HXM_MAX_STREAMS + threadIdx.x] = out_w[threadIdx.x];
+  if (threadIdx.x < S) m[MS * MS + threadIdx.x] = out_w[threadIdx.x];
   __syncthreads();
-  const float* ow = m + HXM_MAX_STREAMS * HXM_MAX_STREAMS;
+  const float* ow = m + MS * MS;
   const int64_t t = blockIdx.x;
   float* xr = x + t * S * W;
   for (int64_t i = threadIdx.x; i < W; i += 256) {
@@ -133,15 +133,15 @@ __global__ __launch_bounds__(256) void stream_update_kernel(float* __restrict__ 
       const float z = A::to_float(gate_pre[t * gate_stride + i]) + (gate_b ? gate_b[i] : 0.f);
       g = g / (1.0f + expf(-z));
     }
-    float old[HXM_MAX_STREAMS];
+    float old[MS];
 #pragma unroll
-    for (int s = 0; s < HXM_MAX_STREAMS; ++s) old[s] = s < S ? xr[s * W + i] : 0.f;
+    for (int s = 0; s < MS; ++s) old[s] = s < S ? xr[s * W + i] : 0.f;
 #pragma unroll
-    for (int d = 0; d < HXM_MAX_STREAMS; ++d) {
+    for (int d = 0; d < MS; ++d) {
       if (d < S) {
         float acc = 0.f;
 #pragma unroll
-        for (int s = 0; s < HXM_MAX_STREAMS; ++s)
+        for (int s = 0; s < MS; ++s)
           if (s < S) acc += m[s * S + d] * old[s];
         xr[d * W + i] = acc + ow[d] * g;
       }
@@ -233,17 +233,18 @@ extern "C" int hxm_stream_update(float* x, const void* y, int64_t y_stride, cons
   if (!x || !y || !mix || !out_w) return HX_ERR_NULL;
   if (y_stride < width || (gate_pre && gate_stride < width)) return HX_ERR_STRIDE;
   hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)n_tokens), block(256);
+#define HXM_UPDATE(A_, T_, MS_) stream_update_kernel<A_, MS_><<<grid, block, 0, s>>>( \
+      x, (const T_*)y, y_stride, (const T_*)gate_pre, gate_stride, gate_b, mix, out_w, n_streams, width)
+#define HXM_UPDATE_MS(A_, T_) do { if (n_streams <= 4) HXM_UPDATE(A_, T_, 4); else if (n_streams <= 8) HXM_UPDATE(A_, T_, 8); \
+      else HXM_UPDATE(A_, T_, 16); } while (0)
   switch (dtype) {
-    case HX_F32:
-      stream_update_kernel<F32><<<dim3((unsigned)n_tokens), dim3(256), 0, s>>>(
-          x, (const float*)y, y_stride, (const float*)gate_pre, gate_stride, gate_b, mix, out_w, n_streams, width);
-      break;
-    case HX_BF16:
-      stream_update_kernel<BF16><<<dim3((unsigned)n_tokens), dim3(256), 0, s>>>(
-          x, (const u16*)y, y_stride, (const u16*)gate_pre, gate_stride, gate_b, mix, out_w, n_streams, width);
-      break;
+    case HX_F32: HXM_UPDATE_MS(F32, float); break;
+    case HX_BF16: HXM_UPDATE_MS(BF16, u16); break;
     default: return HX_ERR_DTYPE;
   }
+#undef HXM_UPDATE_MS
+#undef HXM_UPDATE
   return hxm::check_launch();
 }
 

@@ -55,7 +55,7 @@ def build_node(name: str, node_type: str, language_model, vision_model, lm_shape
             # rows a sequence carries from step to step: one slot per request that can be live at once
             from hydrainfer_amd.memory.state_slots import StateSlotManager
             state = StateSlotManager(sched.max_running_requests, sspec["rows"], sspec["width"], device)
-    if nt.has_image_cache and vision_model is not None:
+    if nt.has_image_cache and n_image_tokens > 0:      # (a text-only model has no image tokens: no pool)
         img = TokenCacheBlockManager(TokenCacheBlockManagerConfig(
             n_layers=1, n_tokens=1, n_blocks=image_blocks, block_size=n_image_tokens,
             n_heads=lm_shape.num_attention_heads, head_size=lm_shape.head_dim, dtype=_DTYPE_NAMES[dtype],

@@ -1,0 +1,217 @@
+"""`bench.py --design tetepel`: prefill and decode throughput of the Tetepel design at sizes that resemble a real model's
+layers (random weights, a few layers), beside the Llama decoder at equal width / feed-forward / heads, and a table of
+the design's own kernels against the Llama path's like kernels, each as a fraction of its roofline (HBM bytes or MFMA
+flops, algorithmic counts).  Both models run their eager step (no captured graph / launch plan) on hand-built batches."""
+import math
+import time
+from typing import Callable, Dict, List
+
+import torch
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0
+
+SIZES = {
+    # width, ff, heads, head dim, latent (kv_rank), query latent, window, streams, norm groups, layers
+    "w2048": dict(width=2048, ff=5632, heads=16, dim=128, kv_rank=256, q_rank=768, window=2048, streams=4, groups=8, layers=4),
+    "w4096": dict(width=4096, ff=11008, heads=32, dim=128, kv_rank=512, q_rank=1536, window=4096, streams=4, groups=8, layers=4),
+}
+VOCAB = 32064
+
+
+def _tetepel(size: dict, dtype, dev):
+    from hydrainfer_amd.model.tetepel import LatentAttentionSpec, TetepelForCausalLM, TetepelLayer, TetepelShape
+    m = LatentAttentionSpec(size["heads"], size["dim"], size["dim"], size["kv_rank"], size["q_rank"],
+                            1.0 / math.sqrt(size["dim"]), size["window"])
+    shape = TetepelShape(VOCAB, size["width"], [TetepelLayer("latent_attention", m, size["ff"]) for _ in range(size["layers"])],
+                         norm_groups=size["groups"], streams=size["streams"], embedding_scale=1.0)
+    return TetepelForCausalLM.random_init(shape, dtype, dev, seed=0)
+
+
+def _llama(size: dict, dtype, dev):
+    from hydrainfer_amd.model.llama import LlamaForCausalLM, LlamaShape
+    shape = LlamaShape(size["width"], size["ff"], size["layers"], size["heads"], size["heads"], size["dim"], VOCAB)
+    return LlamaForCausalLM.random_init(shape, dtype, dev, seed=0)
+
+
+def _batch(model, n_seqs: int, q_len: int, kv_len: int, dtype, dev):
+    """(ids, positions, LanguageModelParameters) of n_seqs sequences that feed their last q_len of kv_len tokens."""
+    from hydrainfer_amd.layer.causal_attention import AttentionParametersBuilder
+    from hydrainfer_amd.memory.kv_cache import KVCache
+    from hydrainfer_amd.model.llama import LanguageModelParameters
+    sh = model.shape
+    bs, nb = 16, (kv_len + 15) // 16
+    b = AttentionParametersBuilder(sh.num_attention_heads, sh.num_key_value_heads, sh.head_dim, bs, dev)
+    for s in range(n_seqs):
+        table = list(range(s * nb, (s + 1) * nb))
+        b.add_request(q_len, kv_len, [table[p // bs] * bs + p % bs for p in range(kv_len - q_len, kv_len)], table)
+    latent = hasattr(model, "cache_spec")
+    for _ in range(sh.num_hidden_layers):
+        k = torch.randn((n_seqs * nb, bs, sh.num_key_value_heads, sh.head_dim), device=dev).to(dtype)
+        b.add_kv_cache(KVCache(k, k if latent else torch.randn_like(k)))
+    ap = b.build_attention_parameters()
+    pos = torch.arange(kv_len - q_len, kv_len, dtype=torch.int32, device=dev).repeat(n_seqs)
+    sel = torch.arange(q_len - 1, n_seqs * q_len, q_len, device=dev)
+    params = LanguageModelParameters(ap, q_len == 1, sel)
+    if latent:
+        from hydrainfer_amd._C.kernel.stream_ops import SequenceState
+        state = torch.zeros((n_seqs, sh.num_hidden_layers, sh.hidden_size), dtype=torch.float32, device=dev)
+        params.sequence_state = SequenceState(state, torch.arange(n_seqs, dtype=torch.int32, device=dev),
+                                              torch.arange(n_seqs, dtype=torch.int32, device=dev).repeat_interleave(q_len))
+    ids = torch.randint(0, VOCAB, (n_seqs * q_len,), device=dev, dtype=torch.int32)
+    return ids, pos, params
+
+
+def _time_eager(fn: Callable, dev, reps: int = 5, warm: int = 2) -> float:
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize(dev)
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        torch.cuda.synchronize(dev)
+        ts.append(time.perf_counter() - t0)
+    return sorted(ts)[len(ts) // 2]
+
+
+def _time_graph(fn: Callable, dev, launches: int = 10, reps: int = 3) -> float:
+    """Microseconds per launch: a hipGraph of `launches` launches, mean of `reps` replays, HIP events."""
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(launches):
+            fn()
+    graph.replay()
+    torch.cuda.synchronize(dev)
+    ts = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(); graph.replay(); e1.record()
+        torch.cuda.synchronize(dev)
+        ts.append(e0.elapsed_time(e1) / launches * 1e3)
+    return sum(ts) / len(ts)
+
+
+def _row(name, us, nbytes=None, flops=None):
+    r = {"kernel": name, "us": round(us, 2)}
+    if nbytes is not None:
+        r.update(bound="hbm", achieved_GBps=round(nbytes / us / 1e3, 1), frac=round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4))
+    else:
+        r.update(bound="mfma", achieved_TFLOPs=round(flops / us / 1e6, 1), frac=round(flops / us / 1e6 / MFMA_PEAK_TFLOPS, 4))
+    return r
+
+
+def throughput(size_name: str, dtype, dev, prefill=(4, 1024), decode=(32, 1024)) -> dict:
+    size = SIZES[size_name]
+    out = {}
+    for name, make in (("tetepel", _tetepel), ("llama", _llama)):
+        model = make(size, dtype, dev)
+        if name == "llama":
+            model.prepare_decode(max_rows=decode[0])
+        with torch.inference_mode():
+            ids, pos, params = _batch(model, prefill[0], prefill[1], prefill[1], dtype, dev)
+            tp = _time_eager(lambda: model(ids, pos, params), dev)
+            ids, pos, params = _batch(model, decode[0], 1, decode[1], dtype, dev)
+            td = _time_eager(lambda: model(ids, pos, params), dev, reps=9, warm=3)
+        out[name] = {"prefill_tok_s": round(prefill[0] * prefill[1] / tp, 1), "prefill_ms": round(tp * 1e3, 3),
+                     "decode_tok_s": round(decode[0] / td, 1), "decode_step_ms": round(td * 1e3, 3),
+                     "weight_GB": round(model.weight_bytes() / 1e9, 3)}
+        del model, params
+        torch.cuda.empty_cache()
+    out["workload"] = {"prefill": f"{prefill[0]} x {prefill[1]} tokens", "decode": f"{decode[0]} sequences at {decode[1]} keys",
+                       "layers": size["layers"], "size": size}
+    return out
+
+
+def kernel_table(size_name: str, dtype, dev, T: int = 4096, n_seqs: int = 4, B: int = 32, ctx: int = 2048) -> dict:
+    """Every kernel of the design at a prefill batch of T tokens (n_seqs portions) — the attention also at a decode batch
+    of B sequences with ctx keys — and the Llama path's like kernels at the same sizes."""
+    from hydrainfer_amd._C.kernel import stream_ops as so
+    from hydrainfer_amd._C.kernel.activation import silu_and_mul
+    from hydrainfer_amd._C.kernel.flash_attn import mha_varlen_fwd
+    from hydrainfer_amd._C.kernel.latent_attn import latent_attention, latent_norm_cache
+    from hydrainfer_amd._C.kernel.norm import add_rms_norm
+    from hydrainfer_amd._C.kernel.position_embedding import rope_set_kv_cache
+    sz = SIZES[size_name]
+    W, S, ff, H, D, R, QR, win = sz["width"], sz["streams"], sz["ff"], sz["heads"], sz["dim"], sz["kv_rank"], sz["q_rank"], sz["window"]
+    e = 2
+    rnd = lambda *s: torch.randn(s, device=dev).to(dtype)
+    f32 = lambda *s: torch.randn(s, device=dev)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev) if not torch.is_tensor(v) else v.to(torch.int32).to(dev)
+    rows: Dict[str, List[dict]] = {"tetepel": [], "llama": []}
+    q_len = T // n_seqs
+    q_cu = i32(list(range(0, T + 1, q_len)))
+    pos = torch.arange(q_len, dtype=torch.int32, device=dev).repeat(n_seqs)
+    tok_seq = torch.arange(n_seqs, dtype=torch.int32, device=dev).repeat_interleave(q_len)
+    x, y, gp = f32(T, S, W), rnd(T, W), rnd(T, W)
+    seq = so.SequenceState(torch.zeros((n_seqs, 1, W), device=dev), i32(list(range(n_seqs))), tok_seq)
+    in_w, nw, shw, gb, mix, ow = f32(S), f32(W), f32(W), f32(W), f32(S, S), f32(S)
+    us = _time_graph(lambda: so.stream_norm(x, in_w, nw, sz["groups"], 1e-6, dtype, shift_w=shw, seq=seq, q_cu=q_cu, positions=pos), dev)
+    rows["tetepel"].append(_row("stream_norm + token shift (reads S streams, writes h and hs)", us, T * W * (4 * S + 2 * e)))
+    us = _time_graph(lambda: so.stream_norm(x, in_w, nw, sz["groups"], 1e-6, dtype), dev)
+    rows["tetepel"].append(_row("stream_norm (feed-forward side)", us, T * W * (4 * S + e)))
+    us = _time_graph(lambda: so.stream_update(x, y, mix, ow, gp, gb), dev)
+    rows["tetepel"].append(_row("stream_update (gated result into S streams)", us, T * W * (8 * S + 2 * e)))
+    gu = rnd(T, 2 * ff)
+    us = _time_graph(lambda: so.gelu_tanh_and_mul(gu[:, :ff], gu[:, ff:]), dev)
+    rows["tetepel"].append(_row("gelu_tanh_and_mul", us, 3 * T * ff * e))
+    nb = (q_len + 15) // 16
+    cache = rnd(n_seqs * nb, 16, 1, R)
+    table, cu_b = i32(torch.randperm(n_seqs * nb)), i32(list(range(0, n_seqs * nb + 1, nb)))
+    slots = i32([int(table[s * nb + p // 16]) * 16 + p % 16 for s in range(n_seqs) for p in range(q_len)])
+    proj = rnd(T, QR + R + H)
+    qw, kw = f32(QR), f32(R)
+    us = _time_graph(lambda: latent_norm_cache(proj, 0, QR, QR, R, qw, kw, 1e-6, slots, cache), dev)
+    rows["tetepel"].append(_row("latent_norm_cache (two norms + cache append)", us, 2 * T * (QR + R) * e))
+    ql = rnd(T, H, R)
+    seen = n_seqs * sum(min(i + 1, win) for i in range(q_len))
+    us = _time_graph(lambda: latent_attention(ql, cache, tok_seq, pos, q_cu, table, cu_b, 1 / math.sqrt(D), win, q_len, gate_pre=proj[:, QR + R:]), dev, launches=4)
+    rows["tetepel"].append(_row(f"latent_attention, prefill {n_seqs} x {q_len} (MFMA tile form, latent {R})", us, flops=4 * H * R * seen))
+    # decode: B sequences, one token each, ctx keys
+    nbd = (ctx + 15) // 16
+    cache_d = rnd(B * nbd, 16, 1, R)
+    table_d, cu_bd = i32(torch.randperm(B * nbd)), i32(list(range(0, B * nbd + 1, nbd)))
+    qd, posd, seqd, qcud = rnd(B, H, R), i32([ctx - 1] * B), i32(list(range(B))), i32(list(range(B + 1)))
+    us = _time_graph(lambda: latent_attention(qd, cache_d, seqd, posd, qcud, table_d, cu_bd, 1 / math.sqrt(D), win, 1), dev)
+    rows["tetepel"].append(_row(f"latent_attention, decode {B} x {min(ctx, win)} keys", us, B * min(ctx, win) * R * e + 2 * B * H * R * e))
+
+    # ---- the Llama path's like kernels
+    res, xx, out, w16 = rnd(T, W), rnd(T, W), rnd(T, W), rnd(W)
+    us = _time_graph(lambda: add_rms_norm(out, res, xx, w16, 1e-6), dev)
+    rows["llama"].append(_row("add_rms_norm (residual add + norm)", us, 4 * T * W * e))
+    us = _time_graph(lambda: silu_and_mul(gu[:, :ff], gu[:, ff:]), dev)
+    rows["llama"].append(_row("silu_and_mul", us, 3 * T * ff * e))
+    q, k, v = rnd(T, H, D), rnd(T, H, D), rnd(T, H, D)
+    kc, vc = rnd(n_seqs * nb, 16, H, D), rnd(n_seqs * nb, 16, H, D)
+    cos_sin = rnd(max(q_len, ctx), 2, D // 2)
+    us = _time_graph(lambda: rope_set_kv_cache(q, k, v, pos, cos_sin, D, slots, kc, vc), dev)
+    rows["llama"].append(_row("rope_set_kv_cache (rotary + cache append)", us, (2 * 2 * T * H * D + 2 * T * H * D) * e))
+    o = torch.empty_like(q)
+    cu_k = q_cu
+    us = _time_graph(lambda: mha_varlen_fwd(o, q, kc, vc, q_cu, cu_k, table, cu_b, None, q_len, q_len, 1 / math.sqrt(D), 0, -1, 0, 0), dev, launches=4)
+    rows["llama"].append(_row(f"mha_varlen_fwd, prefill {n_seqs} x {q_len} (causal, head_dim {D})", us,
+                              flops=4 * H * D * n_seqs * sum(i + 1 for i in range(q_len))))
+    kcd, vcd = rnd(B * nbd, 16, H, D), rnd(B * nbd, 16, H, D)
+    qd2, od2 = rnd(B, H, D), rnd(B, H, D)
+    cu_kd = i32(list(range(0, B * ctx + 1, ctx)))
+    us = _time_graph(lambda: mha_varlen_fwd(od2, qd2, kcd, vcd, qcud, cu_kd, table_d, cu_bd, None, 1, ctx, 1 / math.sqrt(D), 0, -1, 0, 0), dev)
+    rows["llama"].append(_row(f"mha_varlen_fwd, decode {B} x {ctx} keys", us, 2 * B * ctx * H * D * e + 2 * B * H * D * e))
+    rows["workload"] = {"prefill_tokens": T, "portions": n_seqs, "decode_batch": B, "decode_keys": ctx, "size": sz,
+                        "timing": "hipGraph of 10 (attention prefill: 4) launches, mean of 3 replays, HIP events",
+                        "roofline": f"HBM {HBM_PEAK_GBS} GB/s, MFMA {MFMA_PEAK_TFLOPS} TFLOP/s dense bf16; algorithmic bytes / flops"}
+    return rows
+
+
+def run(dtype, dev, sizes=("w2048", "w4096")) -> dict:
+    from hydrainfer_amd import _lib
+    _lib.lib(); _lib.mix_lib()
+    res = {"throughput": {}, "kernels": {}}
+    for s in sizes:
+        res["throughput"][s] = throughput(s, dtype, dev)
+        res["kernels"][s] = kernel_table(s, dtype, dev)
+    return res

@@ -21,8 +21,8 @@ extern "C" {
 #endif
 
 #define HXM_ABI_VERSION 1
-#define HXM_MAX_STREAMS 8
-#define HXM_MAX_LATENT 512      /* widest latent row the attention kernels hold in registers */
+#define HXM_MAX_STREAMS 16
+#define HXM_MAX_LATENT 1024     /* widest latent row the attention kernels hold in registers (the MFMA tile form: 512) */
 
 int hxm_abi_version(void);
 int hxm_last_hip_error(void);
