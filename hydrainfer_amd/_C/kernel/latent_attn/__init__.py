@@ -49,8 +49,9 @@ def latent_norm_cache(proj: Tensor, q_off: int, q_rank: int, kv_off: int, kv_ran
 
 def latent_attention(q: Tensor, cache: Tensor, tok_seq: Tensor, positions: Tensor, q_cu: Tensor, block_table: Tensor,
                      cu_block_lens: Tensor, scale: float, window: Optional[int], max_q_len: int,
-                     gate_pre: Optional[Tensor] = None, out: Optional[Tensor] = None) -> Tensor:
-    """q: [n_tokens, n_heads, kv_rank] (any token / head strides, contiguous rows).  gate_pre [n_tokens, >= n_heads]:
+                     gate_pre: Optional[Tensor] = None, out: Optional[Tensor] = None, max_kv_len: int = 0) -> Tensor:
+    """q: [n_tokens, n_heads, kv_rank] (any token / head strides, contiguous rows).  max_kv_len: the most keys a sequence
+    of the batch holds — lets a launch with few rows (decode steps) deal every row tile's keys to several waves.  gate_pre [n_tokens, >= n_heads]:
     the result of head h is multiplied by sigmoid(gate_pre[t, h]).  Returns [n_tokens, n_heads, kv_rank]."""
     _lib.require_gpu(q, cache, tok_seq, positions, q_cu, block_table, cu_block_lens, gate_pre, out)
     if q.dim() != 3 or q.stride(2) != 1 or cache.dtype != q.dtype:
@@ -85,5 +86,14 @@ def latent_attention(q: Tensor, cache: Tensor, tok_seq: Tensor, positions: Tenso
     a.max_q_len = int(max_q_len)
     a.scale = float(scale)
     a.dtype = _code(q.dtype)
+    a.max_kv_len = int(max_kv_len)      # (0: unknown — no key splits)
+    a.n_splits, a.ws_o, a.ws_ml = 1, None, None
+    if max_kv_len > 0:
+        ns, need = ctypes.c_int32(1), ctypes.c_int64(0)
+        _lib.mix_check(_lib.mix_lib().hxm_latent_attention_plan(ctypes.byref(a), ctypes.byref(ns), ctypes.byref(need)), "latent_attention_plan")
+        if ns.value > 1:
+            ws = torch.empty(need.value, dtype=torch.float32, device=q.device)
+            n_o = need.value // ((R + 15) // 16 * 16 + 2) * ((R + 15) // 16 * 16)
+            a.n_splits, a.ws_o, a.ws_ml = ns.value, ws.data_ptr(), ws.data_ptr() + 4 * n_o
     _lib.mix_check(_lib.mix_lib().hxm_latent_attention(ctypes.byref(a), _lib.current_stream()), "latent_attention")
     return out

@@ -110,6 +110,29 @@ def stream_update(x: Tensor, y: Tensor, mix: Tensor, out_w: Tensor, gate_pre: Op
         _ptr(gate_b), mix.data_ptr(), out_w.data_ptr(), T, S, W, _act_code(y.dtype), _lib.current_stream()), "stream_update")
 
 
+def stream_update_norm(x: Tensor, y: Tensor, mix: Tensor, out_w: Tensor, gate_pre: Optional[Tensor], gate_b: Optional[Tensor],
+                       in_next: Tensor, norm_next: Tensor, groups: int, eps: float) -> Tensor:
+    """stream_update(x, y, mix, out_w, gate_pre, gate_b) and then stream_norm(x, in_next, norm_next, ...) of the next
+    sublayer (one without a token shift), as one launch.  Returns h [n_tokens, width] of y's dtype."""
+    _lib.require_gpu(x, y, mix, out_w, gate_pre, gate_b, in_next, norm_next)
+    _f32(x, "x"); _f32(mix, "mix"); _f32(out_w, "out_w"); _f32(gate_b, "gate_b"); _f32(in_next, "in_next"); _f32(norm_next, "norm_next")
+    T, S, W = x.shape
+    if y.dim() != 2 or y.shape[0] != T or y.shape[1] < W or y.stride(1) != 1:
+        raise _lib.HydraHipError("stream_update_norm: y must be [n_tokens, >= width] with a contiguous last dimension")
+    if gate_pre is not None and (gate_pre.dtype != y.dtype or gate_pre.dim() != 2 or gate_pre.shape[0] != T
+                                 or gate_pre.shape[1] < W or gate_pre.stride(1) != 1):
+        raise _lib.HydraHipError("stream_update_norm: gate_pre must look like y")
+    if mix.numel() != S * S or out_w.numel() != S or in_next.numel() != S or norm_next.numel() != W or \
+            (gate_b is not None and gate_b.numel() != W):
+        raise _lib.HydraHipError("stream_update_norm: mix [S, S], out_w / in_next [S], norm_next / gate_b [width]")
+    h = torch.empty((T, W), dtype=y.dtype, device=x.device)
+    _lib.mix_check(_lib.mix_lib().hxm_stream_update_norm(
+        x.data_ptr(), y.data_ptr(), y.stride(0), _ptr(gate_pre), gate_pre.stride(0) if gate_pre is not None else 0,
+        _ptr(gate_b), mix.data_ptr(), out_w.data_ptr(), in_next.data_ptr(), norm_next.data_ptr(), int(groups), float(eps),
+        h.data_ptr(), T, S, W, _act_code(y.dtype), _lib.current_stream()), "stream_update_norm")
+    return h
+
+
 def gelu_tanh_and_mul(gate: Tensor, up: Tensor) -> Tensor:
     """gelu_tanh(gate) * up in one pass; gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))."""
     _lib.require_gpu(gate, up)

@@ -226,6 +226,7 @@ class hxm_latent_attn_args(ctypes.Structure):
         ("cache_row_stride", c_int64),
         ("n_tokens", c_int32), ("n_seq", c_int32), ("n_heads", c_int32), ("kv_rank", c_int32), ("block_size", c_int32),
         ("window", c_int32), ("max_q_len", c_int32), ("scale", c_float), ("dtype", c_int32),
+        ("max_kv_len", c_int32), ("n_splits", c_int32), ("ws_o", c_void_p), ("ws_ml", c_void_p),
     ]
 
 
@@ -238,10 +239,13 @@ _MIX_SIGNATURES = {
                                 c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "hxm_stream_update": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int32,
                                   c_int64, c_int, c_void_p]),
+    "hxm_stream_update_norm": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                       c_int32, c_float, c_void_p, c_int64, c_int32, c_int64, c_int, c_void_p]),
     "hxm_gelu_tanh_and_mul": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "hxm_latent_norm_cache": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_float, c_void_p,
                                       c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int, c_void_p]),
     "hxm_latent_attention": (c_int, [POINTER(hxm_latent_attn_args), c_void_p]),
+    "hxm_latent_attention_plan": (c_int, [POINTER(hxm_latent_attn_args), POINTER(c_int32), POINTER(c_int64)]),
 }
 
 _mix = None

@@ -24,7 +24,8 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
   return red[0] + red[1] + red[2] + red[3];
 }
 
-// one workgroup per token: both latents of the token from its projection row
+// one workgroup per token: both latents of the token from its projection row.  vec: every pointer, offset and stride
+// lets a lane move four elements at a time.
 template <typename A>
 __global__ __launch_bounds__(256) void latent_norm_cache_kernel(const typename A::storage* __restrict__ proj, int64_t proj_stride,
                                                                 int64_t q_off, int64_t q_rank, int64_t kv_off, int64_t kv_rank,
@@ -32,28 +33,44 @@ __global__ __launch_bounds__(256) void latent_norm_cache_kernel(const typename A
                                                                 typename A::storage* __restrict__ cq_out,
                                                                 const int32_t* __restrict__ slot_ids,
                                                                 typename A::storage* __restrict__ cache, int64_t cache_block_stride,
-                                                                int64_t cache_row_stride, int32_t block_size) {
+                                                                int64_t cache_row_stride, int32_t block_size, int vec) {
   __shared__ float red[4];
+  typedef typename A::storage ST;
+  typedef ST ST4 __attribute__((ext_vector_type(4)));
   const int64_t t = blockIdx.x;
-  const typename A::storage* p = proj + t * proj_stride;
-  float ss = 0.f;
-  for (int64_t i = threadIdx.x; i < q_rank; i += 256) {
-    const float v = A::to_float(p[q_off + i]);
-    ss += v * v;
-  }
-  float inv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)q_rank + eps);
-  for (int64_t i = threadIdx.x; i < q_rank; i += 256)
-    cq_out[t * q_rank + i] = A::from_float(A::to_float(p[q_off + i]) * inv * q_w[i]);
+  const ST* p = proj + t * proj_stride;
   const int32_t slot = slot_ids[t];
-  if (slot < 0) return;
-  ss = 0.f;
-  for (int64_t i = threadIdx.x; i < kv_rank; i += 256) {
-    const float v = A::to_float(p[kv_off + i]);
-    ss += v * v;
+  ST* dst = slot >= 0 ? cache + (int64_t)(slot / block_size) * cache_block_stride + (int64_t)(slot % block_size) * cache_row_stride : nullptr;
+  // the two latents in turn: (source offset, length, weight, destination)
+  for (int which = 0; which < 2; ++which) {
+    const int64_t off = which ? kv_off : q_off, n = which ? kv_rank : q_rank;
+    const float* w = which ? kv_w : q_w;
+    ST* out = which ? dst : cq_out + t * q_rank;
+    if (!out) break;
+    float ss = 0.f;
+    if (vec) {
+      for (int64_t i = 4 * threadIdx.x; i < n; i += 1024) {
+        const ST4 v = *reinterpret_cast<const ST4*>(p + off + i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ss += A::to_float(v[e]) * A::to_float(v[e]);
+      }
+    } else {
+      for (int64_t i = threadIdx.x; i < n; i += 256) ss += A::to_float(p[off + i]) * A::to_float(p[off + i]);
+    }
+    const float inv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)n + eps);
+    if (vec) {
+      for (int64_t i = 4 * threadIdx.x; i < n; i += 1024) {
+        const ST4 v = *reinterpret_cast<const ST4*>(p + off + i);
+        const f32x4 wv = *reinterpret_cast<const f32x4*>(w + i);
+        ST4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = A::from_float(A::to_float(v[e]) * inv * wv[e]);
+        *reinterpret_cast<ST4*>(out + i) = o;
+      }
+    } else {
+      for (int64_t i = threadIdx.x; i < n; i += 256) out[i] = A::from_float(A::to_float(p[off + i]) * inv * w[i]);
+    }
   }
-  inv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)kv_rank + eps);
-  typename A::storage* dst = cache + (int64_t)(slot / block_size) * cache_block_stride + (int64_t)(slot % block_size) * cache_row_stride;
-  for (int64_t i = threadIdx.x; i < kv_rank; i += 256) dst[i] = A::from_float(A::to_float(p[kv_off + i]) * inv * kv_w[i]);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -159,8 +176,11 @@ __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_a
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (wave >= waves_per_block) return;
-  const int64_t item = (int64_t)blockIdx.x * waves_per_block + wave;
-  if (item >= (int64_t)a.n_seq * tiles_per_seq) return;
+  const int n_splits = a.n_splits > 1 ? a.n_splits : 1;
+  const int64_t witem = (int64_t)blockIdx.x * waves_per_block + wave;      // (sequence, row tile, key split), splits fastest
+  if (witem >= (int64_t)a.n_seq * tiles_per_seq * n_splits) return;
+  const int64_t item = witem / n_splits;
+  const int split = (int)(witem % n_splits);
   const int b = (int)(item / tiles_per_seq), tile = (int)(item % tiles_per_seq);
   const int H = a.n_heads, R = a.kv_rank;
   const int q0 = a.q_cu[b];
@@ -220,7 +240,15 @@ __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_a
 #pragma unroll
   for (int n = 0; n < KK * 2; ++n) acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int key0 = k_min; key0 <= k_max; key0 += 32) {
+  // a key split takes a run of whole 32-key chunks of the tile's range (the last splits may get none)
+  int k_begin = k_min, k_end = k_max;
+  if (n_splits > 1) {
+    const int chunks = (k_max - k_min + 32) / 32;
+    const int per = (chunks + n_splits - 1) / n_splits;
+    k_begin = k_min + split * per * 32;
+    k_end = min(k_max, k_begin + per * 32 - 1);
+  }
+  for (int key0 = k_begin; key0 <= k_end; key0 += 32) {
     f32x4 sc[2];
     u16x8 cf[2][KK];
 #pragma unroll
@@ -309,6 +337,25 @@ __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_a
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 
+  if (n_splits > 1) {
+    // unnormalised partial result of this split: ws_o [item][split][16 rows][R16], ws_ml [item][split][16 rows][m, l]
+    float* wo = a.ws_o + ((size_t)witem * 16) * R16;
+    float* wml = a.ws_ml + (size_t)witem * 32;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 4 * g + i;
+      if (c == 0) {
+        wml[2 * row] = m[i];
+        wml[2 * row + 1] = l[i];
+      }
+#pragma unroll
+      for (int n = 0; n < KK * 2; ++n) {
+        const int col = 16 * n + c;
+        if (col < R16) wo[(size_t)row * R16 + col] = acc[n][i];
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = tile * 16 + 4 * g + i;
@@ -328,6 +375,55 @@ __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_a
   }
 }
 
+// the splits of a (sequence, row tile) merged: out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M), times the head gate
+__global__ __launch_bounds__(256) void latent_attn_combine_kernel(hxm_latent_attn_args a, int tiles_per_seq) {
+  const int64_t item = blockIdx.x;
+  const int b = (int)(item / tiles_per_seq), tile = (int)(item % tiles_per_seq);
+  const int H = a.n_heads, R = a.kv_rank, R16 = (R + 15) / 16 * 16, NS = a.n_splits;
+  const int q0 = a.q_cu[b];
+  const int n_rows = (a.q_cu[b + 1] - q0) * H;
+  if (tile * 16 >= n_rows) return;
+  __shared__ float wgt[16][65];      // [row][split] weight e^(m_s - M) / L (NS <= 64)
+  if (threadIdx.x < 16) {
+    const int row = threadIdx.x;
+    const float* wml = a.ws_ml + (size_t)item * NS * 32;
+    float M = -1.0e30f;
+    for (int s = 0; s < NS; ++s) M = fmaxf(M, wml[s * 32 + 2 * row]);
+    float L = 0.f;
+    for (int s = 0; s < NS; ++s) L += wml[s * 32 + 2 * row + 1] * __expf(wml[s * 32 + 2 * row] - M);
+    const int r = tile * 16 + row;
+    float gsc = L > 0.f ? 1.0f / L : 0.f;
+    if (a.gate_pre && r < n_rows) {
+      const float z = BF16::to_float(((const u16*)a.gate_pre)[(int64_t)(q0 + r / H) * a.gate_stride + r % H]);
+      gsc = gsc / (1.0f + __expf(-z));
+    }
+    for (int s = 0; s < NS; ++s) wgt[row][s] = __expf(wml[s * 32 + 2 * row] - M) * gsc;
+  }
+  __syncthreads();
+  const float* wo = a.ws_o + (size_t)item * NS * 16 * R16;
+  for (int e = threadIdx.x; e < 16 * R; e += 256) {
+    const int row = e / R, col = e % R;
+    const int r = tile * 16 + row;
+    if (r >= n_rows) continue;
+    float v = 0.f;
+    for (int s = 0; s < NS; ++s) v += wo[((size_t)s * 16 + row) * R16 + col] * wgt[row][s];
+    ((u16*)a.out)[(int64_t)(q0 + r / H) * a.out_token_stride + (int64_t)(r % H) * a.out_head_stride + col] = BF16::from_float(v);
+  }
+}
+
+// key splits for a launch: enough waves to fill the chip when there are few (sequence, row tile) items — decode steps
+static int tile_splits(const hxm_latent_attn_args& a) {
+  const int tiles_per_seq = (int)(((int64_t)a.max_q_len * a.n_heads + 15) / 16);
+  const int64_t items = (int64_t)a.n_seq * tiles_per_seq;
+  int reach = a.max_kv_len > 0 ? a.max_kv_len : 1;
+  if (a.window > 0 && a.window + a.max_q_len < reach) reach = a.window + a.max_q_len;
+  const int chunks = (reach + 31) / 32;
+  int64_t want = (2048 + items - 1) / items;      // ~8 waves per CU
+  if (want > chunks / 2) want = chunks / 2;          // at least two chunks a split
+  if (want > 64) want = 64;
+  return want < 2 ? 1 : (int)want;
+}
+
 template <int KK>
 int launch_tile(const hxm_latent_attn_args& a, hipStream_t s) {
   const int R16 = (a.kv_rank + 15) / 16 * 16;
@@ -335,9 +431,12 @@ int launch_tile(const hxm_latent_attn_args& a, hipStream_t s) {
   int waves = 4;
   while (waves > 1 && per_wave * waves > 64 * 1024) waves >>= 1;
   const int tiles_per_seq = (int)(((int64_t)a.max_q_len * a.n_heads + 15) / 16);
+  const int n_splits = a.n_splits > 1 ? a.n_splits : 1;
+  if (n_splits > 1 && (n_splits > 64 || !a.ws_o || !a.ws_ml)) return HX_ERR_WORKSPACE;
   const int64_t items = (int64_t)a.n_seq * tiles_per_seq;
-  const dim3 grid((unsigned)((items + waves - 1) / waves));
+  const dim3 grid((unsigned)((items * n_splits + waves - 1) / waves));
   latent_attn_tile_kernel<KK><<<grid, dim3(256), per_wave * waves, s>>>(a, tiles_per_seq, waves);
+  if (n_splits > 1) latent_attn_combine_kernel<<<dim3((unsigned)items), dim3(256), 0, s>>>(a, tiles_per_seq);
   return hxm::check_launch();
 }
 
@@ -352,20 +451,46 @@ extern "C" int hxm_latent_norm_cache(const void* proj, int64_t proj_stride, int6
   if (!proj || !q_w || !kv_w || !cq_out || !slot_ids || !cache) return HX_ERR_NULL;
   if (proj_stride < q_off + q_rank || proj_stride < kv_off + kv_rank || cache_row_stride < kv_rank) return HX_ERR_STRIDE;
   hipStream_t s = (hipStream_t)stream;
+  const int64_t esz = dtype == HX_F32 ? 4 : 2;
+  auto al = [&](const void* q, int64_t bytes) { return (reinterpret_cast<uintptr_t>(q) % bytes) == 0; };
+  const int vec = (q_rank % 4 == 0 && kv_rank % 4 == 0 && q_off % 4 == 0 && kv_off % 4 == 0 && proj_stride % 4 == 0 &&
+                   cache_row_stride % 4 == 0 && cache_block_stride % 4 == 0 && al(proj, 4 * esz) && al(cq_out, 4 * esz) &&
+                   al(cache, 4 * esz) && al(q_w, 16) && al(kv_w, 16)) ? 1 : 0;
   switch (dtype) {
     case HX_F32:
       latent_norm_cache_kernel<F32><<<dim3((unsigned)n_tokens), dim3(256), 0, s>>>(
           (const float*)proj, proj_stride, q_off, q_rank, kv_off, kv_rank, q_w, kv_w, eps, (float*)cq_out, slot_ids,
-          (float*)cache, cache_block_stride, cache_row_stride, block_size);
+          (float*)cache, cache_block_stride, cache_row_stride, block_size, vec);
       break;
     case HX_BF16:
       latent_norm_cache_kernel<BF16><<<dim3((unsigned)n_tokens), dim3(256), 0, s>>>(
           (const u16*)proj, proj_stride, q_off, q_rank, kv_off, kv_rank, q_w, kv_w, eps, (u16*)cq_out, slot_ids,
-          (u16*)cache, cache_block_stride, cache_row_stride, block_size);
+          (u16*)cache, cache_block_stride, cache_row_stride, block_size, vec);
       break;
     default: return HX_ERR_DTYPE;
   }
   return hxm::check_launch();
+}
+
+static bool tile_form_serves(const hxm_latent_attn_args& a) {
+  const bool aligned = a.kv_rank % 8 == 0 && a.cache_row_stride % 8 == 0 && a.cache_block_stride % 8 == 0 &&
+                       a.q_token_stride % 8 == 0 && a.q_head_stride % 8 == 0 && aligned16(a.cache) && aligned16(a.q);
+  return a.dtype == HX_BF16 && aligned && a.kv_rank <= 512 && hxm::tile_form();
+}
+
+extern "C" int hxm_latent_attention_plan(const hxm_latent_attn_args* args, int32_t* n_splits, int64_t* ws_floats) {
+  if (!args || !n_splits || !ws_floats) return HX_ERR_NULL;
+  *n_splits = 1;
+  *ws_floats = 0;
+  if (args->n_tokens <= 0 || args->max_q_len < 1 || args->n_seq < 1 || !tile_form_serves(*args)) return HX_OK;
+  const int ns = tile_splits(*args);
+  if (ns > 1) {
+    const int64_t tiles_per_seq = ((int64_t)args->max_q_len * args->n_heads + 15) / 16;
+    const int64_t R16 = (args->kv_rank + 15) / 16 * 16;
+    *n_splits = ns;
+    *ws_floats = (int64_t)args->n_seq * tiles_per_seq * ns * 16 * (R16 + 2);
+  }
+  return HX_OK;
 }
 
 extern "C" int hxm_latent_attention(const hxm_latent_attn_args* args, void* stream) {
@@ -378,9 +503,7 @@ extern "C" int hxm_latent_attention(const hxm_latent_attn_args* args, void* stre
   if (a.cache_row_stride < a.kv_rank) return HX_ERR_STRIDE;
   hipStream_t s = (hipStream_t)stream;
   if (a.max_q_len < 1) return HX_ERR_SHAPE;
-  const bool aligned = a.kv_rank % 8 == 0 && a.cache_row_stride % 8 == 0 && a.cache_block_stride % 8 == 0 &&
-                       a.q_token_stride % 8 == 0 && a.q_head_stride % 8 == 0 && aligned16(a.cache) && aligned16(a.q);
-  if (a.dtype == HX_BF16 && aligned && a.kv_rank <= 512 && hxm::tile_form()) {
+  if (tile_form_serves(a)) {
     switch ((a.kv_rank + 31) / 32) {
       case 1: return launch_tile<1>(a, s);
       case 2: return launch_tile<2>(a, s);

@@ -19,6 +19,8 @@ def architecture_of(model_path: str) -> str:
     with open(os.path.join(model_path, "config.json")) as f:
         cfg = json.load(f)
     name = cfg.get("architecture") or (cfg.get("architectures") or [None])[0]
+    if name is None and ("text_config" in cfg or "vision_config" in cfg):
+        name = "LlavaForConditionalGeneration"      # a LLaVA configuration written without its class name
     if name is None:
         raise ValueError(f"{model_path}/config.json names no architecture")
     return name

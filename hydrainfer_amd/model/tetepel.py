@@ -34,7 +34,7 @@ from torch import Tensor
 
 from hydrainfer_amd._C.kernel.latent_attn import latent_attention, latent_norm_cache
 from hydrainfer_amd._C.kernel.stream_ops import (SequenceState, gelu_tanh_and_mul, stream_embed, stream_norm,
-                                                  stream_update)
+                                                  stream_update, stream_update_norm)
 
 ARCHITECTURE = "Tetepel"
 
@@ -283,7 +283,9 @@ class TetepelForCausalLM:
         return input_ids
 
     # ------------------------------------------------------------------ forward
-    def _mixer(self, run: int, li: int, x: Tensor, position_ids: Tensor, ap, seq: SequenceState) -> None:
+    def _mixer(self, run: int, li: int, x: Tensor, position_ids: Tensor, ap, seq: SequenceState) -> Optional[Tensor]:
+        """The mixer sublayer of layer run `run`; returns the feed-forward's input when the layer has one (the streams'
+        update and the feed-forward's read side are one launch)."""
         sh, w, m, dt = self.shape, self.lw[li], self.shape.layers[li].mixer, self.dtype
         T, H, D, V, R = x.shape[0], m.heads, m.dim, m.vdim, m.kv_rank
         s1 = w.sub1
@@ -300,16 +302,19 @@ class TetepelForCausalLM:
         o_lat = torch.empty_like(q_lat)
         latent_attention(q_lat.transpose(0, 1), cache, seq.tok_seq, position_ids, ap.q_cu_seq_lens, ap.block_tables,
                          ap.cu_blocks_lens, m.scale, m.window, ap.q_max_seq_len, gate_pre=proj[:, m.q_rank + R:],
-                         out=o_lat.transpose(0, 1))
+                         out=o_lat.transpose(0, 1), max_kv_len=ap.kv_max_seq_len)
         o = torch.bmm(o_lat, w.uv_t)                                          # [H, T, V]
         y = torch.matmul(o.transpose(0, 1).reshape(T, H * V), w.o.t())
         gate_pre = torch.matmul(h, w.rg1.t()) if s1.has_gate else None
+        if w.sub2 is not None:
+            return stream_update_norm(x, y, s1.hc_mix, s1.hc_out, gate_pre, s1.rg_b, w.sub2.hc_in, w.sub2.norm,
+                                      sh.norm_groups, sh.norm_eps)
         stream_update(x, y, s1.hc_mix, s1.hc_out, gate_pre, s1.rg_b)
+        return None
 
-    def _feed_forward(self, li: int, x: Tensor) -> None:
-        sh, w, ff = self.shape, self.lw[li], self.shape.layers[li].ff
+    def _feed_forward(self, li: int, x: Tensor, h: Tensor) -> None:
+        w, ff = self.lw[li], self.shape.layers[li].ff
         s2 = w.sub2
-        h = stream_norm(x, s2.hc_in, s2.norm, sh.norm_groups, sh.norm_eps, self.dtype)
         gu = torch.matmul(h, w.w_ff.t())                                      # [T, gate | up | result gate]
         act = gelu_tanh_and_mul(gu[:, :ff], gu[:, ff:2 * ff])
         y = torch.matmul(act, w.down.t())
@@ -335,9 +340,9 @@ class TetepelForCausalLM:
             seq = SequenceState(None, None, tok_seq)
         x = stream_embed(input_ids.contiguous(), self.embed_table, sh.embedding_scale, sh.streams)
         for run, li in enumerate(sh.run_order):
-            self._mixer(run, li, x, position_ids, model_params.attention_params[run], seq)
+            h_ff = self._mixer(run, li, x, position_ids, model_params.attention_params[run], seq)
             if sh.layers[li].ff:
-                self._feed_forward(li, x)
+                self._feed_forward(li, x, h_ff)
             if self.layer_trace is not None:
                 self.layer_trace.append(x.sum(dim=1))
         sel = model_params.selected_token_ids

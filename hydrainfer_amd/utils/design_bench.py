@@ -170,14 +170,14 @@ def kernel_table(size_name: str, dtype, dev, T: int = 4096, n_seqs: int = 4, B: 
     rows["tetepel"].append(_row("latent_norm_cache (two norms + cache append)", us, 2 * T * (QR + R) * e))
     ql = rnd(T, H, R)
     seen = n_seqs * sum(min(i + 1, win) for i in range(q_len))
-    us = _time_graph(lambda: latent_attention(ql, cache, tok_seq, pos, q_cu, table, cu_b, 1 / math.sqrt(D), win, q_len, gate_pre=proj[:, QR + R:]), dev, launches=4)
+    us = _time_graph(lambda: latent_attention(ql, cache, tok_seq, pos, q_cu, table, cu_b, 1 / math.sqrt(D), win, q_len, gate_pre=proj[:, QR + R:], max_kv_len=q_len), dev, launches=4)
     rows["tetepel"].append(_row(f"latent_attention, prefill {n_seqs} x {q_len} (MFMA tile form, latent {R})", us, flops=4 * H * R * seen))
     # decode: B sequences, one token each, ctx keys
     nbd = (ctx + 15) // 16
     cache_d = rnd(B * nbd, 16, 1, R)
     table_d, cu_bd = i32(torch.randperm(B * nbd)), i32(list(range(0, B * nbd + 1, nbd)))
     qd, posd, seqd, qcud = rnd(B, H, R), i32([ctx - 1] * B), i32(list(range(B))), i32(list(range(B + 1)))
-    us = _time_graph(lambda: latent_attention(qd, cache_d, seqd, posd, qcud, table_d, cu_bd, 1 / math.sqrt(D), win, 1), dev)
+    us = _time_graph(lambda: latent_attention(qd, cache_d, seqd, posd, qcud, table_d, cu_bd, 1 / math.sqrt(D), win, 1, max_kv_len=ctx), dev)
     rows["tetepel"].append(_row(f"latent_attention, decode {B} x {min(ctx, win)} keys", us, B * min(ctx, win) * R * e + 2 * B * H * R * e))
 
     # ---- the Llama path's like kernels

@@ -57,6 +57,13 @@ int hxm_stream_update(float* x, const void* y, int64_t y_stride, const void* gat
                       const float* gate_b, const float* mix, const float* out_w, int64_t n_tokens, int32_t n_streams,
                       int64_t width, int dtype, void* stream);
 
+/* hxm_stream_update followed by the read side of the NEXT sublayer (one without a token shift) in one launch: the streams
+ * are updated in place and h_out [n_tokens, width] = grouped_rms_norm(sum_s in_next[s] * x_new[., s, :]) * norm_next. */
+int hxm_stream_update_norm(float* x, const void* y, int64_t y_stride, const void* gate_pre, int64_t gate_stride,
+                           const float* gate_b, const float* mix, const float* out_w, const float* in_next,
+                           const float* norm_next, int32_t groups, float eps, void* h_out, int64_t n_tokens,
+                           int32_t n_streams, int64_t width, int dtype, void* stream);
+
 /* out[., i] = gelu_tanh(gate[., i]) * up[., i], gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))). */
 int hxm_gelu_tanh_and_mul(void* out, const void* gate, const void* up, int64_t rows, int64_t n, int64_t gate_stride,
                           int64_t up_stride, int dtype, void* stream);
@@ -87,7 +94,16 @@ typedef struct hxm_latent_attn_args {
   int32_t max_q_len;         /* the longest portion of the batch (1: every sequence decodes) */
   float scale;
   int32_t dtype;
+  int32_t max_kv_len;        /* the most keys a sequence of the batch holds (sizes the key splits) */
+  int32_t n_splits;          /* from hxm_latent_attention_plan; > 1: the key range of a row tile is dealt to n_splits waves */
+  float* ws_o;               /* n_splits > 1: the plan's workspace, ws_floats floats; ws_ml = where its (max, sum) pairs go */
+  float* ws_ml;
 } hxm_latent_attn_args;
+
+/* How a launch with these arguments would be laid out: n_splits (1: no workspace) and the floats of workspace it needs
+ * (ws_o = the first n_items * n_splits * 16 * ceil16(kv_rank) of them, ws_ml = the rest).  Pointers need not be set yet,
+ * except q and cache (their alignment decides the form). */
+int hxm_latent_attention_plan(const hxm_latent_attn_args* args, int32_t* n_splits, int64_t* ws_floats);
 
 /* Softmax attention of every query over the latents of its own sequence in the paged cache (scores and weights in
  * float).  Queries of portions and single decoded tokens may share a batch. */

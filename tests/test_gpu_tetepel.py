@@ -17,6 +17,16 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+@pytest.fixture(autouse=True)
+def _leave_the_device_rng_alone():
+    """Cache pools are filled from the device's default generator; tests that come after this file keep drawing the
+    numbers they drew before it existed."""
+    state = torch.cuda.get_rng_state(DEV) if torch.cuda.is_available() else None
+    yield
+    if state is not None:
+        torch.cuda.set_rng_state(state, DEV)
+
+
 def _shape(kind: str):
     from hydrainfer_amd.model.tetepel import LatentAttentionSpec as A, TetepelLayer as L, TetepelShape
     if kind == "looped":        # three streams, grouped norm, a looped span, windows that differ, a layer without feed-forward
@@ -110,7 +120,7 @@ TOL32, TOL16 = 2e-4, 5e-2
 def test_stream_embed_norm_update_and_gelu_kernels():
     from hydrainfer_amd._C.kernel import stream_ops as so
     g = torch.Generator().manual_seed(1)
-    for S, W_, groups in ((1, 40, 1), (3, 96, 4), (5, 136, 8), (8, 48, 3)):
+    for S, W_, groups in ((1, 40, 1), (3, 96, 4), (5, 136, 8), (8, 48, 3), (4, 1024, 2), (2, 512, 1), (16, 768, 3), (3, 46, 2)):
         T = 9
         table = torch.randn(30, W_, generator=g)
         ids = torch.randint(0, 30, (T,), generator=g)
@@ -131,6 +141,14 @@ def test_stream_embed_norm_update_and_gelu_kernels():
         ref = oracle.streams_write(x.double().transpose(0, 1), y.double() * torch.sigmoid(gp[:, :W_].double() + gb.double()),
                                    mix.double(), w_out.double()).transpose(0, 1)
         _close(xd.cpu(), ref, 1e-5, "stream_update gated")
+        # the update and the next sublayer's read side as one launch
+        xd = x.to(DEV).clone()
+        in2, nw2 = torch.randn(S, generator=g), torch.randn(W_, generator=g)
+        h2 = so.stream_update_norm(xd, y.to(DEV), mix.to(DEV), w_out.to(DEV), gp.to(DEV)[:, :W_], gb.to(DEV), in2.to(DEV), nw2.to(DEV),
+                                   groups, 1e-5)
+        _close(xd.cpu(), ref, 1e-5, "stream_update_norm: streams")
+        _close(h2.cpu(), oracle.grouped_rms_norm(oracle.streams_read(ref.transpose(0, 1), in2.double()), nw2.double(), groups, 1e-5),
+               1e-5, "stream_update_norm: h")
         xd = x.to(DEV).clone()
         so.stream_update(xd, y.to(DEV), mix.to(DEV), w_out.to(DEV))
         _close(xd.cpu(), oracle.streams_write(x.double().transpose(0, 1), y.double(), mix.double(), w_out.double()).transpose(0, 1),
@@ -142,12 +160,13 @@ def test_stream_embed_norm_update_and_gelu_kernels():
     _close(out16.float().cpu(), oracle.gelu_tanh(a.bfloat16().double()) * b.bfloat16().double(), 2e-2, "gelu bf16")
 
 
-def test_token_shift_carries_the_previous_row_through_the_state_slot():
+@pytest.mark.parametrize("W_,groups", [(48, 4), (768, 3), (50, 5)])
+def test_token_shift_carries_the_previous_row_through_the_state_slot(W_, groups):
     """Two sequences in one batch, cut into portions (one of a single token, one of two): the shifted rows equal the
     shift of the whole sequences, the slot of a reused sequence number starts from zeros at position 0."""
     from hydrainfer_amd._C.kernel import stream_ops as so
     g = torch.Generator().manual_seed(2)
-    S, W_, groups = 2, 48, 4
+    S = 2
     lens = {0: 9, 1: 6}
     xs = {b: torch.randn(n, S, W_, generator=g) for b, n in lens.items()}
     w_in, nw, sh = torch.randn(S, generator=g), torch.randn(W_, generator=g), torch.rand(W_, generator=g)
@@ -228,20 +247,20 @@ def test_latent_attention_kernel_window_edges_page_borders_and_far_keys(R, H, wi
         ch = cache.to(dtype)
         qd = q[idx].to(dtype).to(DEV)
         out = latent_attention(qd, ch, tok_seq[idx].to(DEV), positions[idx].to(DEV), q_cu.to(DEV), table, cu_blocks, scale,
-                               window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV))
+                               window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV), max_kv_len=max(n_ctx))
         _close(out.float().cpu(), ref[idx], tol, f"latent attention {dtype}")
         # strided query / result layouts (heads outermost), as the model hands them over
         qh = qd.transpose(0, 1).contiguous()
         oh = torch.empty_like(qh)
         latent_attention(qh.transpose(0, 1), ch, tok_seq[idx].to(DEV), positions[idx].to(DEV), q_cu.to(DEV), table, cu_blocks,
-                         scale, window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV), out=oh.transpose(0, 1))
+                         scale, window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV), out=oh.transpose(0, 1), max_kv_len=max(n_ctx))
         assert torch.equal(oh.transpose(0, 1), out)
         if dtype == torch.bfloat16:      # the row form of the same kernel (what float32 runs on) agrees with the tile form
             from hydrainfer_amd import _lib
             _lib.mix_lib().hxm_set_option(b"attn_tile_form", 0)
             try:
                 rows = latent_attention(qd, ch, tok_seq[idx].to(DEV), positions[idx].to(DEV), q_cu.to(DEV), table, cu_blocks,
-                                        scale, window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV))
+                                        scale, window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV), max_kv_len=max(n_ctx))
             finally:
                 _lib.mix_lib().hxm_set_option(b"attn_tile_form", 1)
             _close(rows.float().cpu(), ref[idx], tol, "latent attention, row form in bfloat16")
@@ -397,3 +416,55 @@ def test_registry_loads_a_checkpoint_directory(tmp_path):
     toks = _tokens(20, shape.vocab_size, 9)
     got = _run(_replayer(lm, torch.float32, 32), {"a": toks}, [[("a", 20)]])["a"]
     _close(got, oracle.forward(shape.to_config(), W, toks), TOL32, "loaded checkpoint")
+
+
+def test_trace_run_command_line(tmp_path):
+    """bin/trace_run as a user starts it: steps on standard input, `done <step>` lines and .f32 files out."""
+    import json
+    import subprocess
+    import numpy as np
+    import safetensors.torch
+    shape = _shape("looped")
+    W = _weights(shape, seed=18)
+    model_dir, out_dir = tmp_path / "model", tmp_path / "out"
+    model_dir.mkdir()
+    (model_dir / "config.json").write_text(json.dumps(shape.to_config()))
+    safetensors.torch.save_file({k: v.to(torch.bfloat16) for k, v in W.items()}, str(model_dir / "model.safetensors"))
+    a, b = _tokens(21, shape.vocab_size, 40), _tokens(9, shape.vocab_size, 41)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:17], "want": [0, 16]}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[:8], "want": []}, {"id": "a", "tokens": a[17:18], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[18:], "want": [2]}, {"id": "b", "tokens": b[8:], "want": [0]}], "end": ["a", "b"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", str(model_dir), "--dtype", "float32", "--out", str(out_dir),
+                        "--max-tokens", "64"], input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    ra, rb = oracle.forward(shape.to_config(), W, a), oracle.forward(shape.to_config(), W, b)
+    read = lambda n: torch.from_numpy(np.fromfile(str(out_dir / f"{n}.f32"), dtype="<f4")).view(-1, shape.vocab_size)
+    _close(read(0), ra[[0, 16]], TOL32, "step 0")
+    _close(read(1), ra[[17]], TOL32, "step 1")
+    _close(read(2), torch.cat([ra[[20]], rb[[8]]]), TOL32, "step 2")
+
+
+@pytest.mark.parametrize("lens", [(1500, 700, 100), (3000, 1201, 50, 1)])
+def test_token_shift_in_long_batches(lens):
+    """Thousands of rows in one launch: a workgroup then takes several consecutive rows and hands h from one to the next;
+    sequence borders fall inside such runs."""
+    from hydrainfer_amd._C.kernel import stream_ops as so
+    g = torch.Generator().manual_seed(7)
+    S, W_, groups = 3, 56, 7
+    xs = [torch.randn(n, S, W_, generator=g) for n in lens]
+    w_in, nw, sh = torch.randn(S, generator=g), torch.randn(W_, generator=g), torch.rand(W_, generator=g)
+    norm = lambda x: oracle.grouped_rms_norm(oracle.streams_read(x.double().transpose(0, 1), w_in.double()), nw.double(), groups, 1e-6)
+    ref = torch.cat([oracle.token_shift(norm(x), sh.double()) for x in xs])
+    state = torch.zeros((len(lens), 1, W_), device=DEV)
+    q_cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    pos = torch.cat([torch.arange(n) for n in lens]).to(torch.int32)
+    tok_seq = torch.cat([torch.full((n,), i) for i, n in enumerate(lens)]).to(torch.int32)
+    seq = so.SequenceState(state, torch.arange(len(lens), dtype=torch.int32, device=DEV), tok_seq.to(DEV))
+    h, hs = so.stream_norm(torch.cat(xs).to(DEV), w_in.to(DEV), nw.to(DEV), groups, 1e-6, torch.float32, shift_w=sh.to(DEV), seq=seq,
+                           q_cu=q_cu.to(DEV), positions=pos.to(DEV))
+    _close(hs.cpu(), ref, 1e-5, "shifted rows")
+    _close(h.cpu(), torch.cat([norm(x) for x in xs]), 1e-5, "plain rows")
+    _close(state[:, 0].cpu(), torch.stack([norm(x)[-1] for x in xs]), 1e-5, "state rows: the h of every sequence's last token")
