@@ -165,11 +165,13 @@ __global__ __launch_bounds__(256) void latent_attn_rows_kernel(hxm_latent_attn_a
 // sixteen heads of a decoded token, or a few tokens times a few heads.  All rows of a tile read the same keys, which go
 // by in chunks of 32: S = Q C^T and O += P C are 16x16x32 MFMAs.  The chunk's rows come straight from the paged cache
 // into the B operands of S (a lane's 16 bytes are 8 consecutive columns of one key's row); for O the same registers are
-// written to the wave's LDS transposed (CT[column][key], two keys a word), P goes through LDS from the accumulator
-// layout to the A layout.  Inside a chunk the 32 keys are summed in the order slot = 2 * (key % 16) + key / 16 in both
-// operands, so that a lane's two keys are neighbours.  No barriers: a wave shares nothing with its neighbours.
+// written to the wave's LDS as they are (row-major image of the chunk, 16 bytes a write) and come back through the
+// transposing LDS read (ds_read_b64_tr_b16: a lane gets one column of four rows) as B operands; P goes through LDS from
+// the accumulator layout to the A layout.  Inside a chunk the 32 keys are summed in the order the transposing read
+// delivers them — lane group g: keys 4g .. 4g+3, then 16+4g .. 16+4g+3 — in both operands.  No workgroup barriers: a wave
+// shares nothing with its neighbours.
 // ---------------------------------------------------------------------------------------------------------------
-constexpr int kCtStride = 36;      // u16 per CT / P row: 32 slots + 4 (72 bytes: the four 16-lane groups of a write hit different banks)
+constexpr int kPStride = 36;       // u16 per row of P in LDS: 32 slots + 4
 
 template <int KK>                  // ceil(kv_rank / 32), 1 .. 16
 __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_args a, int tiles_per_seq, int waves_per_block) {
@@ -188,8 +190,9 @@ __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_a
   if (tile * 16 >= n_rows) return;
   const int g = lane >> 4, c = lane & 15;
   const int R16 = (R + 15) / 16 * 16;
-  u16* ct = reinterpret_cast<u16*>(lds) + (size_t)wave * (R16 + 16) * kCtStride;
-  u16* pl = ct + (size_t)R16 * kCtStride;
+  const int RS = 2 * (KK * 32) + 32;      // bytes per row of the chunk's image (a key's columns, padded)
+  char* img = reinterpret_cast<char*>(lds) + (size_t)wave * (32 * RS + 16 * kPStride * 2);
+  u16* pl = reinterpret_cast<u16*>(img + 32 * RS);
   const u16* cache = (const u16*)a.cache;
   const int32_t* table = a.block_table + a.cu_block_lens[b];
 
@@ -265,17 +268,12 @@ __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_a
         sc[s] = Mfma<BF16>::mma(qf[kk], cf[s][kk], sc[s]);
       }
     }
-    // the chunk, transposed, for the second product: CT[column][slot], slot = 2 c + s
+    // the chunk's image for the second product: row = key 16 s + c, the lane's eight columns as they came
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) {
-      const int col = 32 * kk + 8 * g;
-      if (col < R) {
+    for (int s = 0; s < 2; ++s)
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-          *reinterpret_cast<uint32_t*>(ct + (size_t)(col + j) * kCtStride + 2 * c) =
-              (uint32_t)cf[0][kk][j] | ((uint32_t)cf[1][kk][j] << 16);
-      }
-    }
+      for (int kk = 0; kk < KK; ++kk)
+        *reinterpret_cast<u16x8*>(img + (16 * s + c) * RS + (32 * kk + 8 * g) * 2) = cf[s][kk];
     // softmax of the rows 4 g + i over this chunk (sc[s][i] is key key0 + 16 s + c)
     float p[2][4];
 #pragma unroll
@@ -309,25 +307,26 @@ __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_a
       m[i] = m_new;
 #pragma unroll
       for (int n = 0; n < KK * 2; ++n) acc[n][i] *= corr;
-      *reinterpret_cast<uint32_t*>(pl + (size_t)(4 * g + i) * kCtStride + 2 * c) =
-          (uint32_t)BF16::from_float(p[0][i]) | ((uint32_t)BF16::from_float(p[1][i]) << 16);
+      // key 16 s + c sits in slot 8 (c / 4) + c % 4 + 4 s of its row
+      pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3)] = BF16::from_float(p[0][i]);
+      pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3) + 4] = BF16::from_float(p[1][i]);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // O += P C: A = P[row c][slots 8 g ..], B = CT[column 16 n + c][slots 8 g ..]
+    // O += P C: A = P[row c][slots 8 g ..], B = the image's column 16 n + c at the keys of those slots
     u16x8 pf;
     {
-      const u16x4 x0 = *reinterpret_cast<const u16x4*>(pl + (size_t)c * kCtStride + 8 * g);
-      const u16x4 x1 = *reinterpret_cast<const u16x4*>(pl + (size_t)c * kCtStride + 8 * g + 4);
+      const u16x4 x0 = *reinterpret_cast<const u16x4*>(pl + c * kPStride + 8 * g);
+      const u16x4 x1 = *reinterpret_cast<const u16x4*>(pl + c * kPStride + 8 * g + 4);
       pf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
     }
+    const char* vrd = img + (4 * g + (c >> 2)) * RS + (c & 3) * 8;
 #pragma unroll
     for (int n = 0; n < KK * 2; ++n) {
       if (16 * n < R) {
-        const u16* src = ct + (size_t)(16 * n + c) * kCtStride + 8 * g;
-        const u16x4 x0 = *reinterpret_cast<const u16x4*>(src);
-        const u16x4 x1 = *reinterpret_cast<const u16x4*>(src + 4);
+        const u16x4 x0 = lds_tr_read(vrd + n * 32);
+        const u16x4 x1 = lds_tr_read(vrd + 16 * RS + n * 32);
         const u16x8 vf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
         acc[n] = Mfma<BF16>::mma(pf, vf, acc[n]);
       }
@@ -426,8 +425,7 @@ static int tile_splits(const hxm_latent_attn_args& a) {
 
 template <int KK>
 int launch_tile(const hxm_latent_attn_args& a, hipStream_t s) {
-  const int R16 = (a.kv_rank + 15) / 16 * 16;
-  const size_t per_wave = (size_t)(R16 + 16) * kCtStride * sizeof(u16);
+  const size_t per_wave = (size_t)32 * (2 * (KK * 32) + 32) + 16 * kPStride * 2;
   int waves = 4;
   while (waves > 1 && per_wave * waves > 64 * 1024) waves >>= 1;
   const int tiles_per_seq = (int)(((int64_t)a.max_q_len * a.n_heads + 15) / 16);
@@ -435,7 +433,7 @@ int launch_tile(const hxm_latent_attn_args& a, hipStream_t s) {
   if (n_splits > 1 && (n_splits > 64 || !a.ws_o || !a.ws_ml)) return HX_ERR_WORKSPACE;
   const int64_t items = (int64_t)a.n_seq * tiles_per_seq;
   const dim3 grid((unsigned)((items * n_splits + waves - 1) / waves));
-  latent_attn_tile_kernel<KK><<<grid, dim3(256), per_wave * waves, s>>>(a, tiles_per_seq, waves);
+  latent_attn_tile_kernel<KK><<<grid, dim3(64 * waves), per_wave * waves, s>>>(a, tiles_per_seq, waves);
   if (n_splits > 1) latent_attn_combine_kernel<<<dim3((unsigned)items), dim3(256), 0, s>>>(a, tiles_per_seq);
   return hxm::check_launch();
 }
