@@ -24,8 +24,8 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
   return red[0] + red[1] + red[2] + red[3];
 }
 
-// one workgroup per token: both latents of the token from its projection row.  vec: every pointer, offset and stride
-// lets a lane move four elements at a time.
+// one WAVE per token (four tokens a workgroup, no barriers): both latents of the token from its projection row.  vec:
+// every pointer, offset and stride lets a lane move four elements at a time.
 template <typename A>
 __global__ __launch_bounds__(256) void latent_norm_cache_kernel(const typename A::storage* __restrict__ proj, int64_t proj_stride,
                                                                 int64_t q_off, int64_t q_rank, int64_t kv_off, int64_t kv_rank,
@@ -33,11 +33,12 @@ __global__ __launch_bounds__(256) void latent_norm_cache_kernel(const typename A
                                                                 typename A::storage* __restrict__ cq_out,
                                                                 const int32_t* __restrict__ slot_ids,
                                                                 typename A::storage* __restrict__ cache, int64_t cache_block_stride,
-                                                                int64_t cache_row_stride, int32_t block_size, int vec) {
-  __shared__ float red[4];
+                                                                int64_t cache_row_stride, int32_t block_size, int64_t n_tokens, int vec) {
   typedef typename A::storage ST;
   typedef ST ST4 __attribute__((ext_vector_type(4)));
-  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= n_tokens) return;
   const ST* p = proj + t * proj_stride;
   const int32_t slot = slot_ids[t];
   ST* dst = slot >= 0 ? cache + (int64_t)(slot / block_size) * cache_block_stride + (int64_t)(slot % block_size) * cache_row_stride : nullptr;
@@ -49,17 +50,17 @@ __global__ __launch_bounds__(256) void latent_norm_cache_kernel(const typename A
     if (!out) break;
     float ss = 0.f;
     if (vec) {
-      for (int64_t i = 4 * threadIdx.x; i < n; i += 1024) {
+      for (int64_t i = 4 * lane; i < n; i += 256) {
         const ST4 v = *reinterpret_cast<const ST4*>(p + off + i);
 #pragma unroll
         for (int e = 0; e < 4; ++e) ss += A::to_float(v[e]) * A::to_float(v[e]);
       }
     } else {
-      for (int64_t i = threadIdx.x; i < n; i += 256) ss += A::to_float(p[off + i]) * A::to_float(p[off + i]);
+      for (int64_t i = lane; i < n; i += 64) ss += A::to_float(p[off + i]) * A::to_float(p[off + i]);
     }
-    const float inv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)n + eps);
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)n + eps);
     if (vec) {
-      for (int64_t i = 4 * threadIdx.x; i < n; i += 1024) {
+      for (int64_t i = 4 * lane; i < n; i += 256) {
         const ST4 v = *reinterpret_cast<const ST4*>(p + off + i);
         const f32x4 wv = *reinterpret_cast<const f32x4*>(w + i);
         ST4 o;
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(256) void latent_norm_cache_kernel(const typename A
         *reinterpret_cast<ST4*>(out + i) = o;
       }
     } else {
-      for (int64_t i = threadIdx.x; i < n; i += 256) out[i] = A::from_float(A::to_float(p[off + i]) * inv * w[i]);
+      for (int64_t i = lane; i < n; i += 64) out[i] = A::from_float(A::to_float(p[off + i]) * inv * w[i]);
     }
   }
 }
@@ -251,6 +252,239 @@ __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_a
     k_begin = k_min + split * per * 32;
     k_end = min(k_max, k_begin + per * 32 - 1);
   }
+  const int bs = a.block_size;
+  const int bshift = (bs & (bs - 1)) == 0 ? __ffs(bs) - 1 : -1;
+  // half a chunk's rows, this lane's part: key 16 s + c, columns 32 kk + 8 g .. + 7
+  auto fetch = [&](int key0, int s, u16x8 (&cf)[KK]) __attribute__((always_inline)) {
+    const int key = min(key0 + 16 * s + c, k_max);        // (a key past the last one repeats it; masked below)
+    const int page = bshift >= 0 ? key >> bshift : key / bs;
+    const u16* row = cache + (int64_t)table[page] * a.cache_block_stride + (int64_t)(key - page * bs) * a.cache_row_stride;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int col = 32 * kk + 8 * g;
+      if (col < R) cf[kk] = *reinterpret_cast<const u16x8*>(row + col);
+      else cf[kk] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  };
+  // scores of half a chunk, and its rows into the image for the second product (row = key 16 s + c, the lane's eight
+  // columns as they came)
+  auto score = [&](int s, const u16x8 (&cf)[KK]) __attribute__((always_inline)) -> f32x4 {
+    f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      v = Mfma<BF16>::mma(qf[kk], cf[kk], v);
+      *reinterpret_cast<u16x8*>(img + (16 * s + c) * RS + (32 * kk + 8 * g) * 2) = cf[kk];
+    }
+    return v;
+  };
+  auto finish = [&](int key0, const f32x4 (&sc)[2]) __attribute__((always_inline)) {
+    // softmax of the rows 4 g + i over this chunk (sc[s][i] is key key0 + 16 s + c)
+    float p[2][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const int key = key0 + 16 * s + c;
+        const bool seen = key >= lo[i] && key <= pos[i];
+        const float v = seen ? sc[s][i] * a.scale : -INFINITY;
+        p[s][i] = v;
+        mx = fmaxf(mx, v);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
+      const float m_new = fmaxf(m[i], mx);
+      const float corr = __expf(m[i] - m_new);
+      float ps = 0.f;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        p[s][i] = __expf(p[s][i] - m_new);       // exp(-inf) = 0 for a key the row does not see
+        ps += p[s][i];
+      }
+      ps += __shfl_xor(ps, 1, 64);
+      ps += __shfl_xor(ps, 2, 64);
+      ps += __shfl_xor(ps, 4, 64);
+      ps += __shfl_xor(ps, 8, 64);
+      l[i] = l[i] * corr + ps;
+      m[i] = m_new;
+#pragma unroll
+      for (int n = 0; n < KK * 2; ++n) acc[n][i] *= corr;
+      // key 16 s + c sits in slot 8 (c / 4) + c % 4 + 4 s of its row
+      pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3)] = BF16::from_float(p[0][i]);
+      pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3) + 4] = BF16::from_float(p[1][i]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // O += P C: A = P[row c][slots 8 g ..], B = the image's column 16 n + c at the keys of those slots
+    u16x8 pf;
+    {
+      const u16x4 x0 = *reinterpret_cast<const u16x4*>(pl + c * kPStride + 8 * g);
+      const u16x4 x1 = *reinterpret_cast<const u16x4*>(pl + c * kPStride + 8 * g + 4);
+      pf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+    }
+    const char* vrd = img + (4 * g + (c >> 2)) * RS + (c & 3) * 8;
+#pragma unroll
+    for (int n = 0; n < KK * 2; ++n) {
+      {      // (column tiles past the latent's width read zeros of the image: no branch around an MFMA)
+        const u16x4 x0 = lds_tr_read(vrd + n * 32);
+        const u16x4 x1 = lds_tr_read(vrd + 16 * RS + n * 32);
+        const u16x8 vf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        acc[n] = Mfma<BF16>::mma(pf, vf, acc[n]);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();      // the reads are done before the next chunk is written
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  {
+    // two register sets: the next chunk's rows are on their way while this one is worked on
+    u16x8 ca[2][KK], cb[2][KK];
+    f32x4 sc[2];
+    if (k_begin <= k_end) {
+      fetch(k_begin, 0, ca[0]);
+      fetch(k_begin, 1, ca[1]);
+    }
+    for (int key0 = k_begin; key0 <= k_end; key0 += 64) {
+      const bool more = key0 + 32 <= k_end;
+      if (more) {
+        fetch(key0 + 32, 0, cb[0]);
+        fetch(key0 + 32, 1, cb[1]);
+      }
+      sc[0] = score(0, ca[0]);
+      sc[1] = score(1, ca[1]);
+      finish(key0, sc);
+      if (more) {
+        if (key0 + 64 <= k_end) {
+          fetch(key0 + 64, 0, ca[0]);
+          fetch(key0 + 64, 1, ca[1]);
+        }
+        sc[0] = score(0, cb[0]);
+        sc[1] = score(1, cb[1]);
+        finish(key0 + 32, sc);
+      }
+    }
+  }
+  if (n_splits > 1) {
+    // unnormalised partial result of this split: ws_o [item][split][16 rows][R16], ws_ml [item][split][16 rows][m, l]
+    float* wo = a.ws_o + ((size_t)witem * 16) * R16;
+    float* wml = a.ws_ml + (size_t)witem * 32;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 4 * g + i;
+      if (c == 0) {
+        wml[2 * row] = m[i];
+        wml[2 * row + 1] = l[i];
+      }
+#pragma unroll
+      for (int n = 0; n < KK * 2; ++n) {
+        const int col = 16 * n + c;
+        if (col < R16) wo[(size_t)row * R16 + col] = acc[n][i];
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 16 + 4 * g + i;
+    if (r >= n_rows) continue;
+    const int t = q0 + r / H, h = r % H;
+    float gsc = 1.0f / l[i];
+    if (a.gate_pre) {
+      const float z = BF16::to_float(((const u16*)a.gate_pre)[(int64_t)t * a.gate_stride + h]);
+      gsc = gsc / (1.0f + __expf(-z));
+    }
+    u16* og = (u16*)a.out + (int64_t)t * a.out_token_stride + (int64_t)h * a.out_head_stride;
+#pragma unroll
+    for (int n = 0; n < KK * 2; ++n) {
+      const int col = 16 * n + c;
+      if (col < R) og[col] = BF16::from_float(acc[n][i] * gsc);
+    }
+  }
+}
+
+// The same for latents of more than 256 columns: no second register set for the rows on their way (the accumulators
+// and the queries leave no room), a whole chunk in registers between its two products.
+template <int KK>                  // ceil(kv_rank / 32), 9 .. 16
+__global__ __launch_bounds__(256) void latent_attn_tile_wide_kernel(hxm_latent_attn_args a, int tiles_per_seq, int waves_per_block) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (wave >= waves_per_block) return;
+  const int n_splits = a.n_splits > 1 ? a.n_splits : 1;
+  const int64_t witem = (int64_t)blockIdx.x * waves_per_block + wave;      // (sequence, row tile, key split), splits fastest
+  if (witem >= (int64_t)a.n_seq * tiles_per_seq * n_splits) return;
+  const int64_t item = witem / n_splits;
+  const int split = (int)(witem % n_splits);
+  const int b = (int)(item / tiles_per_seq), tile = (int)(item % tiles_per_seq);
+  const int H = a.n_heads, R = a.kv_rank;
+  const int q0 = a.q_cu[b];
+  const int n_rows = (a.q_cu[b + 1] - q0) * H;
+  if (tile * 16 >= n_rows) return;
+  const int g = lane >> 4, c = lane & 15;
+  const int R16 = (R + 15) / 16 * 16;
+  const int RS = 2 * (KK * 32) + 32;      // bytes per row of the chunk's image (a key's columns, padded)
+  char* img = reinterpret_cast<char*>(lds) + (size_t)wave * (32 * RS + 16 * kPStride * 2);
+  u16* pl = reinterpret_cast<u16*>(img + 32 * RS);
+  const u16* cache = (const u16*)a.cache;
+  const int32_t* table = a.block_table + a.cu_block_lens[b];
+
+  // the queries: lane (g, c) holds row c, columns 32 kk + 8 g .. + 7
+  const int last_row = min(tile * 16 + 15, n_rows - 1);
+  u16x8 qf[KK];
+  {
+    const int r = min(tile * 16 + c, n_rows - 1);
+    const u16* qg = (const u16*)a.q + (int64_t)(q0 + r / H) * a.q_token_stride + (int64_t)(r % H) * a.q_head_stride;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int col = 32 * kk + 8 * g;
+      if (col < R) qf[kk] = *reinterpret_cast<const u16x8*>(qg + col);
+      else qf[kk] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+  // the rows this lane holds of S and O: 4 g + i
+  int pos[4], lo[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 16 + 4 * g + i;
+    if (r < n_rows) {
+      pos[i] = a.positions[q0 + r / H];
+      lo[i] = a.window > 0 ? max(0, pos[i] - a.window + 1) : 0;
+    } else {
+      pos[i] = -1;      // sees nothing
+      lo[i] = 0;
+    }
+  }
+  // the keys any row of the tile sees: lane (., c) looks at row c, the sixteen are reduced by shuffles
+  int k_min, k_max;
+  {
+    const int r = min(tile * 16 + c, last_row);
+    const int pr = a.positions[q0 + r / H];
+    k_max = pr;
+    k_min = a.window > 0 ? max(0, pr - a.window + 1) : 0;
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+      k_max = max(k_max, __shfl_xor(k_max, off, 64));
+      k_min = min(k_min, __shfl_xor(k_min, off, 64));
+    }
+  }
+
+  float m[4], l[4];
+  f32x4 acc[KK * 2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { m[i] = -1.0e30f; l[i] = 0.f; }
+#pragma unroll
+  for (int n = 0; n < KK * 2; ++n) acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // a key split takes a run of whole 32-key chunks of the tile's range (the last splits may get none)
+  int k_begin = k_min, k_end = k_max;
+  if (n_splits > 1) {
+    const int chunks = (k_max - k_min + 32) / 32;
+    const int per = (chunks + n_splits - 1) / n_splits;
+    k_begin = k_min + split * per * 32;
+    k_end = min(k_max, k_begin + per * 32 - 1);
+  }
   for (int key0 = k_begin; key0 <= k_end; key0 += 32) {
     f32x4 sc[2];
     u16x8 cf[2][KK];
@@ -324,7 +558,7 @@ __global__ __launch_bounds__(256) void latent_attn_tile_kernel(hxm_latent_attn_a
     const char* vrd = img + (4 * g + (c >> 2)) * RS + (c & 3) * 8;
 #pragma unroll
     for (int n = 0; n < KK * 2; ++n) {
-      if (16 * n < R) {
+      {      // (column tiles past the latent's width read zeros of the image: no branch around an MFMA)
         const u16x4 x0 = lds_tr_read(vrd + n * 32);
         const u16x4 x1 = lds_tr_read(vrd + 16 * RS + n * 32);
         const u16x8 vf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
@@ -433,7 +667,8 @@ int launch_tile(const hxm_latent_attn_args& a, hipStream_t s) {
   if (n_splits > 1 && (n_splits > 64 || !a.ws_o || !a.ws_ml)) return HX_ERR_WORKSPACE;
   const int64_t items = (int64_t)a.n_seq * tiles_per_seq;
   const dim3 grid((unsigned)((items * n_splits + waves - 1) / waves));
-  latent_attn_tile_kernel<KK><<<grid, dim3(64 * waves), per_wave * waves, s>>>(a, tiles_per_seq, waves);
+  if constexpr (KK <= 8) latent_attn_tile_kernel<KK><<<grid, dim3(64 * waves), per_wave * waves, s>>>(a, tiles_per_seq, waves);
+  else latent_attn_tile_wide_kernel<KK><<<grid, dim3(64 * waves), per_wave * waves, s>>>(a, tiles_per_seq, waves);
   if (n_splits > 1) latent_attn_combine_kernel<<<dim3((unsigned)items), dim3(256), 0, s>>>(a, tiles_per_seq);
   return hxm::check_launch();
 }
@@ -456,14 +691,14 @@ extern "C" int hxm_latent_norm_cache(const void* proj, int64_t proj_stride, int6
                    al(cache, 4 * esz) && al(q_w, 16) && al(kv_w, 16)) ? 1 : 0;
   switch (dtype) {
     case HX_F32:
-      latent_norm_cache_kernel<F32><<<dim3((unsigned)n_tokens), dim3(256), 0, s>>>(
+      latent_norm_cache_kernel<F32><<<dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, s>>>(
           (const float*)proj, proj_stride, q_off, q_rank, kv_off, kv_rank, q_w, kv_w, eps, (float*)cq_out, slot_ids,
-          (float*)cache, cache_block_stride, cache_row_stride, block_size, vec);
+          (float*)cache, cache_block_stride, cache_row_stride, block_size, n_tokens, vec);
       break;
     case HX_BF16:
-      latent_norm_cache_kernel<BF16><<<dim3((unsigned)n_tokens), dim3(256), 0, s>>>(
+      latent_norm_cache_kernel<BF16><<<dim3((unsigned)((n_tokens + 3) / 4)), dim3(256), 0, s>>>(
           (const u16*)proj, proj_stride, q_off, q_rank, kv_off, kv_rank, q_w, kv_w, eps, (u16*)cq_out, slot_ids,
-          (u16*)cache, cache_block_stride, cache_row_stride, block_size, vec);
+          (u16*)cache, cache_block_stride, cache_row_stride, block_size, n_tokens, vec);
       break;
     default: return HX_ERR_DTYPE;
   }
