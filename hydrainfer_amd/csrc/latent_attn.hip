@@ -15,15 +15,6 @@ namespace {
 
 using namespace hx;
 
-__device__ __forceinline__ float block_sum_256(float v, float* red) {
-  v = wave_sum(v);
-  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  __syncthreads();
-  if (lane == 0) red[wid] = v;
-  __syncthreads();
-  return red[0] + red[1] + red[2] + red[3];
-}
-
 // one WAVE per token (four tokens a workgroup, no barriers): both latents of the token from its projection row.  vec:
 // every pointer, offset and stride lets a lane move four elements at a time.
 template <typename A>
