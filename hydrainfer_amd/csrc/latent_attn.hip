@@ -599,6 +599,185 @@ __global__ __launch_bounds__(256) void latent_attn_tile_wide_kernel(hxm_latent_a
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Group form (bfloat16, portions of prompts): a workgroup of four waves takes four consecutive row tiles (64 rows) of a
+// sequence and ONE image of every 32-key chunk: each wave brings eight of the chunk's rows from the paged cache into
+// LDS, then all four read their B operands of both products from there (16-byte reads for S, transposing reads for O).
+// Against the tile form: a quarter of the global reads and LDS writes per wave, and no registers spent on the chunk.
+// Two workgroup barriers a chunk (image complete / image free).  Used for latents of more than 256 columns.
+// ---------------------------------------------------------------------------------------------------------------
+template <int KK>
+__global__ __launch_bounds__(256) void latent_attn_group_kernel(hxm_latent_attn_args a, int groups_per_seq) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t item = blockIdx.x;      // (sequence, group of four row tiles)
+  const int b = (int)(item / groups_per_seq), grp = (int)(item % groups_per_seq);
+  const int H = a.n_heads, R = a.kv_rank;
+  const int q0 = a.q_cu[b];
+  const int n_rows = (a.q_cu[b + 1] - q0) * H;
+  if (grp * 64 >= n_rows) return;       // (the whole workgroup)
+  const int tile = grp * 4 + wave;
+  const bool live = tile * 16 < n_rows; // a wave without rows still brings its share of every chunk
+  const int g = lane >> 4, c = lane & 15;
+  const int RS = 2 * (KK * 32) + 32;    // bytes per row of the chunk's image (a key's columns, padded)
+  char* img = reinterpret_cast<char*>(lds);
+  u16* pl = reinterpret_cast<u16*>(img + 32 * RS) + wave * 16 * kPStride;
+  const u16* cache = (const u16*)a.cache;
+  const int32_t* table = a.block_table + a.cu_block_lens[b];
+  // the image's columns past the latent's width stay zero (the loads below never touch them)
+  for (int i = threadIdx.x; i < 2 * RS; i += 256) reinterpret_cast<u16x8*>(img)[i] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+
+  u16x8 qf[KK];
+  {
+    const int r = min(tile * 16 + c, n_rows - 1);
+    const u16* qg = (const u16*)a.q + (int64_t)(q0 + r / H) * a.q_token_stride + (int64_t)(r % H) * a.q_head_stride;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int col = 32 * kk + 8 * g;
+      if (col < R) qf[kk] = *reinterpret_cast<const u16x8*>(qg + col);
+      else qf[kk] = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+  int pos[4], lo[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 16 + 4 * g + i;
+    if (r < n_rows) {
+      pos[i] = a.positions[q0 + r / H];
+      lo[i] = a.window > 0 ? max(0, pos[i] - a.window + 1) : 0;
+    } else {
+      pos[i] = -1;      // sees nothing
+      lo[i] = 0;
+    }
+  }
+  // the keys any row of the GROUP sees (the same in every wave): lane l looks at row 64 grp + l
+  int k_min, k_max;
+  {
+    const int r = min(grp * 64 + lane, n_rows - 1);
+    const int pr = a.positions[q0 + r / H];
+    k_max = pr;
+    k_min = a.window > 0 ? max(0, pr - a.window + 1) : 0;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      k_max = max(k_max, __shfl_xor(k_max, off, 64));
+      k_min = min(k_min, __shfl_xor(k_min, off, 64));
+    }
+  }
+  float m[4], l[4];
+  f32x4 acc[KK * 2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { m[i] = -1.0e30f; l[i] = 0.f; }
+#pragma unroll
+  for (int n = 0; n < KK * 2; ++n) acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int bs = a.block_size;
+  const int bshift = (bs & (bs - 1)) == 0 ? __ffs(bs) - 1 : -1;
+  auto finish = [&](int key0, const f32x4 (&sc)[2]) __attribute__((always_inline)) {
+    // softmax of the rows 4 g + i over this chunk (sc[s][i] is key key0 + 16 s + c)
+    float p[2][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const int key = key0 + 16 * s + c;
+        const bool seen = key >= lo[i] && key <= pos[i];
+        const float v = seen ? sc[s][i] * a.scale : -INFINITY;
+        p[s][i] = v;
+        mx = fmaxf(mx, v);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
+      const float m_new = fmaxf(m[i], mx);
+      const float corr = __expf(m[i] - m_new);
+      float ps = 0.f;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        p[s][i] = __expf(p[s][i] - m_new);       // exp(-inf) = 0 for a key the row does not see
+        ps += p[s][i];
+      }
+      ps += __shfl_xor(ps, 1, 64);
+      ps += __shfl_xor(ps, 2, 64);
+      ps += __shfl_xor(ps, 4, 64);
+      ps += __shfl_xor(ps, 8, 64);
+      l[i] = l[i] * corr + ps;
+      m[i] = m_new;
+#pragma unroll
+      for (int n = 0; n < KK * 2; ++n) acc[n][i] *= corr;
+      // key 16 s + c sits in slot 8 (c / 4) + c % 4 + 4 s of its row
+      pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3)] = BF16::from_float(p[0][i]);
+      pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3) + 4] = BF16::from_float(p[1][i]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // O += P C: A = P[row c][slots 8 g ..], B = the image's column 16 n + c at the keys of those slots
+    u16x8 pf;
+    {
+      const u16x4 x0 = *reinterpret_cast<const u16x4*>(pl + c * kPStride + 8 * g);
+      const u16x4 x1 = *reinterpret_cast<const u16x4*>(pl + c * kPStride + 8 * g + 4);
+      pf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+    }
+    const char* vrd = img + (4 * g + (c >> 2)) * RS + (c & 3) * 8;
+#pragma unroll
+    for (int n = 0; n < KK * 2; ++n) {
+      {      // (column tiles past the latent's width read zeros of the image: no branch around an MFMA)
+        const u16x4 x0 = lds_tr_read(vrd + n * 32);
+        const u16x4 x1 = lds_tr_read(vrd + 16 * RS + n * 32);
+        const u16x8 vf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        acc[n] = Mfma<BF16>::mma(pf, vf, acc[n]);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();      // the reads are done before the next chunk is written
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  __syncthreads();      // the zeroed image
+  for (int key0 = k_min; key0 <= k_max; key0 += 32) {
+    // this wave's eight rows of the chunk: key0 + 8 wave + kq, a lane brings eight columns
+#pragma unroll
+    for (int kq = 0; kq < 8; ++kq) {
+      const int key = min(key0 + 8 * wave + kq, k_max);      // (a key past the last one repeats it; masked in the softmax)
+      const int page = bshift >= 0 ? key >> bshift : key / bs;
+      const u16* row = cache + (int64_t)table[page] * a.cache_block_stride + (int64_t)(key - page * bs) * a.cache_row_stride;
+      for (int col = lane * 8; col < R; col += 512)
+        *reinterpret_cast<u16x8*>(img + (8 * wave + kq) * RS + col * 2) = *reinterpret_cast<const u16x8*>(row + col);
+    }
+    __syncthreads();      // the image is complete
+    if (live) {
+      f32x4 sc[2];
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        sc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk)
+          sc[s] = Mfma<BF16>::mma(qf[kk], *reinterpret_cast<const u16x8*>(img + (16 * s + c) * RS + (32 * kk + 8 * g) * 2), sc[s]);
+      }
+      finish(key0, sc);
+    }
+    __syncthreads();      // every wave is done with the image
+  }
+  if (!live) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 16 + 4 * g + i;
+    if (r >= n_rows) continue;
+    const int t = q0 + r / H, h = r % H;
+    float gsc = 1.0f / l[i];
+    if (a.gate_pre) {
+      const float z = BF16::to_float(((const u16*)a.gate_pre)[(int64_t)t * a.gate_stride + h]);
+      gsc = gsc / (1.0f + __expf(-z));
+    }
+    u16* og = (u16*)a.out + (int64_t)t * a.out_token_stride + (int64_t)h * a.out_head_stride;
+#pragma unroll
+    for (int n = 0; n < KK * 2; ++n) {
+      const int col = 16 * n + c;
+      if (col < R) og[col] = BF16::from_float(acc[n][i] * gsc);
+    }
+  }
+}
+
 // the splits of a (sequence, row tile) merged: out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M), times the head gate
 __global__ __launch_bounds__(256) void latent_attn_combine_kernel(hxm_latent_attn_args a, int tiles_per_seq) {
   const int64_t item = blockIdx.x;
@@ -656,6 +835,14 @@ int launch_tile(const hxm_latent_attn_args& a, hipStream_t s) {
   const int tiles_per_seq = (int)(((int64_t)a.max_q_len * a.n_heads + 15) / 16);
   const int n_splits = a.n_splits > 1 ? a.n_splits : 1;
   if (n_splits > 1 && (n_splits > 64 || !a.ws_o || !a.ws_ml)) return HX_ERR_WORKSPACE;
+  // (measured: the group form wins where the tile form has no room for its second register set — latents of more than 256
+  //  columns: 1136 -> 891 us at 512 columns — and loses below: 89 -> 140 us at 64 columns)
+  if (KK > 8 && n_splits == 1 && tiles_per_seq >= 4 && hxm::tile_form() == 1) {
+    const int groups_per_seq = (tiles_per_seq + 3) / 4;
+    const size_t lds_g = (size_t)32 * (2 * (KK * 32) + 32) + 4 * 16 * kPStride * 2;
+    latent_attn_group_kernel<KK><<<dim3((unsigned)((int64_t)a.n_seq * groups_per_seq)), dim3(256), lds_g, s>>>(a, groups_per_seq);
+    return hxm::check_launch();
+  }
   const int64_t items = (int64_t)a.n_seq * tiles_per_seq;
   const dim3 grid((unsigned)((items * n_splits + waves - 1) / waves));
   if constexpr (KK <= 8) latent_attn_tile_kernel<KK><<<grid, dim3(64 * waves), per_wave * waves, s>>>(a, tiles_per_seq, waves);

@@ -396,7 +396,7 @@ extern "C" int hxm_abi_version(void) { return HXM_ABI_VERSION; }
 extern "C" int hxm_last_hip_error(void) { return hxm::last_hip_error(); }
 extern "C" int hxm_set_option(const char* name, int value) {
   if (name && __builtin_strcmp(name, "attn_tile_form") == 0) {
-    hxm::tile_form() = value ? 1 : 0;
+    hxm::tile_form() = value < 0 ? 0 : value > 2 ? 2 : value;
     return HX_OK;
   }
   return HX_ERR_UNSUPPORTED;

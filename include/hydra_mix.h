@@ -27,7 +27,8 @@ extern "C" {
 int hxm_abi_version(void);
 int hxm_last_hip_error(void);
 /* A/B measurements in one process: "attn_tile_form" = 0 keeps bfloat16 attention on the row form (one wave per token
- * and head) instead of the MFMA tile form.  Results agree within bfloat16 rounding. */
+ * and head) instead of the MFMA forms, 2 keeps portions of prompts on the tile form (one wave per 16 rows) instead of
+ * the group form (four waves sharing every chunk of keys), 1 = the default.  Results agree within bfloat16 rounding. */
 int hxm_set_option(const char* name, int value);
 
 /* x[t, s, :] = table[ids[t], :] * scale for every stream s.  x: float [n_tokens, n_streams, width]; table: dtype

@@ -208,8 +208,8 @@ def _paged(c_rows, block_size, row_width, seed, dtype=torch.float32):
     return cache.to(dtype).to(DEV), torch.tensor(table, dtype=torch.int32, device=DEV), torch.tensor(cu, dtype=torch.int32, device=DEV)
 
 
-@pytest.mark.parametrize("R,H,window", [(40, 3, 17), (128, 4, 96), (320, 2, None), (64, 1, 1), (72, 5, 16), (48, 2, 9), (104, 4, 40),
-                                            (80, 3, None), (200, 2, 64), (8, 16, 5), (112, 1, 300)])
+@pytest.mark.parametrize("R,H,window", [(40, 3, 17), (128, 8, 100), (320, 2, None), (64, 1, 1), (72, 5, 16), (48, 2, 9), (104, 4, 40),
+                                            (80, 3, None), (200, 2, 64), (8, 16, 5), (112, 1, 300), (328, 3, 29), (512, 2, None)])
 def test_latent_attention_kernel_window_edges_page_borders_and_far_keys(R, H, window):
     """One key is made to stand out (the query is a multiple of its row): just inside the window, just outside it, on
     both sides of a page border, and the sequence's first key hundreds of positions back."""
@@ -254,6 +254,10 @@ def test_latent_attention_kernel_window_edges_page_borders_and_far_keys(R, H, wi
         out = latent_attention(qd, ch, tok_seq[idx].to(DEV), positions[idx].to(DEV), q_cu.to(DEV), table, cu_blocks, scale,
                                window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV), max_kv_len=max(n_ctx))
         _close(out.float().cpu(), ref[idx], tol, f"latent attention {dtype}")
+        # without key splits (no bound on the keys given): wide latents then take the group form, four waves a chunk
+        whole = latent_attention(qd, ch, tok_seq[idx].to(DEV), positions[idx].to(DEV), q_cu.to(DEV), table, cu_blocks, scale,
+                                 window, int(q_cu.diff().max()), gate_pre=gate[idx].to(dtype).to(DEV))
+        _close(whole.float().cpu(), ref[idx], tol, f"latent attention {dtype}, no key splits")
         # strided query / result layouts (heads outermost), as the model hands them over
         qh = qd.transpose(0, 1).contiguous()
         oh = torch.empty_like(qh)

@@ -114,3 +114,20 @@ def test_registry_names_the_architecture(tmp_path):
     (tmp_path / "config.json").write_text(json.dumps({"architectures": ["Nope"]}))
     with pytest.raises(ValueError):
         load_model(str(tmp_path), torch.float32, "cpu")
+
+
+def test_mix_library_exports_what_its_header_declares():
+    """include/hydra_mix.h, the ctypes table and the built library name the same entry points (no GPU needed to open it)."""
+    import ctypes
+    import os
+    import re
+    from hydrainfer_amd import _lib
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    declared = set(re.findall(r"^(?:int|int64_t|const char\*)\s+(hxm_\w+)\(", open(os.path.join(root, "include", "hydra_mix.h")).read(), re.M))
+    assert declared == set(_lib._MIX_SIGNATURES), declared ^ set(_lib._MIX_SIGNATURES)
+    if not os.path.exists(_lib.MIX_LIB_PATH):
+        pytest.skip("libhydra_mix.so is not built")
+    handle = ctypes.CDLL(_lib.MIX_LIB_PATH)
+    for name in declared:
+        assert hasattr(handle, name), name
+    assert handle.hxm_abi_version() == _lib.HXM_ABI_VERSION
