@@ -41,6 +41,10 @@ def _shape(kind: str):
     if kind == "wide":          # latents wider than 64 / 128 / 256 columns, five streams, whole model looped
         return TetepelShape(130, 128, [L("latent_attention", A(2, 32, 16, 320, 48, 0.2, 33), 64)],
                             loop_start=0, loop_stop=1, loop_times=3, norm_eps=1e-6, norm_groups=8, streams=5, embedding_scale=0.5)
+    if kind == "odd":           # nothing a multiple of four: every kernel's element-by-element path, the row-form attention
+        return TetepelShape(45, 38, [L("latent_attention", A(3, 6, 10, 20, 10, 0.35, 5), 26),
+                                     L("latent_attention", A(2, 5, 3, 9, 7, 0.6, None), 13)],
+                            loop_start=0, loop_stop=2, loop_times=2, norm_eps=1e-4, norm_groups=2, streams=2, embedding_scale=1.5)
     raise KeyError(kind)
 
 
@@ -296,14 +300,15 @@ def test_latent_norm_cache_kernel_writes_the_rows_it_is_told_to():
 
 
 # ------------------------------------------------------------------------------------------------ the model in the engine
-@pytest.mark.parametrize("kind", ["looped", "plain", "wide"])
+@pytest.mark.parametrize("kind", ["looped", "plain", "wide", "odd"])
 def test_whole_prompts_match_the_oracle_layer_by_layer(kind):
     shape = _shape(kind)
     W = _weights(shape, seed=11)
     toks = _tokens(70, shape.vocab_size, 4)
     sums = []
     ref = oracle.forward(shape.to_config(), W, toks, sums)
-    for dtype, tol in ((torch.float32, TOL32), (torch.bfloat16, TOL16)):
+    # (bfloat16 rounding averages out over fewer terms in 9-column latents and 19-element norm groups)
+    for dtype, tol in ((torch.float32, TOL32), (torch.bfloat16, 8e-2 if kind == "odd" else TOL16)):
         lm = _model(shape, W, dtype)
         rp = _replayer(lm, dtype, 128)
         lm.language_model.layer_trace = []
@@ -327,7 +332,7 @@ def test_checkpoint_without_shift_gates_and_stream_weights():
     _close(got, ref, TOL32, "no shift / gates / stream weights")
 
 
-@pytest.mark.parametrize("kind", ["looped", "wide"])
+@pytest.mark.parametrize("kind", ["looped", "wide", "odd"])
 def test_decoding_token_by_token_and_portions_of_every_size_equal_the_whole_prompt(kind):
     shape = _shape(kind)
     W = _weights(shape, seed=13)
