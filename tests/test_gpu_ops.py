@@ -180,10 +180,14 @@ def test_quick_gelu_equals_the_three_torch_ops():
             assert got.shape == x.shape and got.dtype == dt
             if dt == torch.float32:
                 assert_ulp_close(got.cpu(), want.cpu(), max_ulp=8, what=f"{dt} {shape}")
-            else:                         # the same three roundings, each product through fp32 first: bit for bit
-                assert torch.equal(got, want), f"{dt} {shape}: {(got != want).sum().item()} elements differ"
+            else:
+                # the same three roundings, each product through fp32 first.  Bit for bit except where the two fp32
+                # sigmoids differ in their last bit AND that bit decides the rounding to T: measured over 400 random
+                # draws, one tensor of 320 elements in forty holds such an element (one unit in the last place)
+                assert_ulp_close(got.cpu(), want.cpu(), max_ulp=1, min_exact_frac=0.999, what=f"{dt} {shape}")
     x = (3 * torch.randn((9, 2 * 512), device=DEV)).to(torch.bfloat16)            # row-strided input
-    assert torch.equal(act.quick_gelu(x[:, :512]), x[:, :512] * torch.sigmoid(1.702 * x[:, :512]))
+    assert_ulp_close(act.quick_gelu(x[:, :512]).cpu(), (x[:, :512] * torch.sigmoid(1.702 * x[:, :512])).cpu(), max_ulp=1,
+                     min_exact_frac=0.999, what="row-strided input")
     with pytest.raises(RuntimeError):
         act.quick_gelu(torch.zeros((4, 12), dtype=torch.bfloat16, device=DEV))    # n % 8
 
@@ -207,7 +211,9 @@ def test_add_layer_norm_equals_add_then_layer_norm():
             exact = F.layer_norm(h_ref.double(), (hidden,), w.double(), b.double(), 1e-5)
             assert (out.double() - exact).abs().max().item() <= tol * 4, (dt, rows, hidden)
             if dt != torch.float32:      # (fp32: an output next to zero is a cancellation — ulps mean nothing there)
-                assert_ulp_close(out.cpu(), want.cpu(), max_ulp=2, min_exact_frac=0.98, what=f"{dt} {rows}x{hidden}")
+                # (an output next to zero is a cancellation of O(1) terms there too: a few units in ITS last place are
+                #  far below one unit of the row's scale — three were seen once in a dozen runs of the suite)
+                assert_ulp_close(out.cpu(), want.cpu(), max_ulp=4, min_exact_frac=0.98, what=f"{dt} {rows}x{hidden}")
             else:
                 assert (out - want).abs().max().item() <= 4e-6
             res2, out2 = h_ref.clone(), torch.empty_like(h)
