@@ -64,8 +64,10 @@ def main():
     ApiServer(front, tok, ClipImageProcessor(), host=a.host, port=a.port).run()
 
 
-def serve_checkpoint(a, dt, dev):
-    """One collocated replica of the model in a checkpoint directory, whatever registered architecture it is."""
+def build_checkpoint_server(a, dt, dev):
+    """(ApiServer, EngineFrontend) around one collocated replica of the model in the checkpoint directory a.checkpoint,
+    whatever registered architecture it is.  a: the parsed command line (checkpoint, max_running, max_tokens, tokenizer,
+    host, port)."""
     from hydrainfer_amd.engine.node import LocalCluster
     from hydrainfer_amd.engine.request_processor import InstructionCreator
     from hydrainfer_amd.engine.scheduler import BatchSchedulerConfig
@@ -85,10 +87,17 @@ def serve_checkpoint(a, dt, dev):
                       image_blocks=2 * a.max_running, n_image_tokens=n_img, sched=sched, max_blocks_per_seq=per_req)
     creator = InstructionCreator(image_token_id=lm.image_token_id, n_image_tokens_per_image=n_img, block_size=16,
                                  max_position_embeddings=shape.max_position_embeddings, prefix_cache=not stateful)
-    tok = HFTokenizer(a.tokenizer) if a.tokenizer else SyntheticTokenizer(image_token_id=lm.image_token_id)
+    # (no tokenizer files offline: the synthetic one hashes words into the model's own vocabulary)
+    tok = HFTokenizer(a.tokenizer) if a.tokenizer else SyntheticTokenizer(image_token_id=lm.image_token_id, lo=min(3, shape.vocab_size - 1),
+                                                                           hi=min(31999, shape.vocab_size))
     front = EngineFrontend(LocalCluster([node]), creator, device=dev)
+    return ApiServer(front, tok, ClipImageProcessor() if vision is not None else None, host=a.host, port=a.port), front
+
+
+def serve_checkpoint(a, dt, dev):
+    server, _ = build_checkpoint_server(a, dt, dev)
     print(f"serving {a.checkpoint} ({a.dtype}) on http://{a.host}:{a.port}/v1/chat/completions", flush=True)
-    ApiServer(front, tok, ClipImageProcessor(), host=a.host, port=a.port).run()
+    server.run()
 
 
 if __name__ == "__main__":

@@ -482,3 +482,40 @@ def test_token_shift_in_long_batches(lens):
     _close(hs.cpu(), ref, 1e-5, "shifted rows")
     _close(h.cpu(), torch.cat([norm(x) for x in xs]), 1e-5, "plain rows")
     _close(state[:, 0].cpu(), torch.stack([norm(x)[-1] for x in xs]), 1e-5, "state rows: the h of every sequence's last token")
+
+
+def test_chat_endpoint_serves_a_checkpoint_directory(tmp_path):
+    """`python -m hydrainfer_amd.entrypoint --checkpoint DIR` in parts: registry -> node -> front end -> HTTP endpoint.  The
+    streams carry the tokens the offline engine generates for the same token ids."""
+    import asyncio
+    import json
+    from types import SimpleNamespace
+    import safetensors.torch
+    from hydrainfer_amd.engine.offline import OfflineInferenceEngine, OfflineRequest
+    from hydrainfer_amd.entrypoint.__main__ import build_checkpoint_server
+    from tests.test_api_server import _client_stream, _payload
+    shape = _shape("looped")
+    W = _weights(shape, seed=19)
+    (tmp_path / "config.json").write_text(json.dumps(shape.to_config()))
+    safetensors.torch.save_file({k: v.to(torch.bfloat16) for k, v in W.items()}, str(tmp_path / "model.safetensors"))
+    args = SimpleNamespace(checkpoint=str(tmp_path), max_running=4, max_tokens=128, tokenizer=None, host="127.0.0.1", port=0, dtype="fp32")
+    server, front = build_checkpoint_server(args, torch.float32, torch.device(DEV))
+    jobs = [("what a fine day it is today", 6), ("one two three four five six seven eight nine ten eleven twelve", 9), ("hello", 4)]
+
+    async def go():
+        await server.start()
+        front.start()
+        try:
+            return await asyncio.gather(*[_client_stream(f"http://127.0.0.1:{server.port}/v1", _payload(t, None, n)) for t, n in jobs])
+        finally:
+            front.stop()
+            await server.close()
+    got = asyncio.run(go())
+    assert front.error is None and front.n_admitted == len(jobs)
+    from hydrainfer_amd.entrypoint.api_protocol import parse_chat_completion_request as parse
+    eng = OfflineInferenceEngine.from_checkpoint(str(tmp_path), torch.float32, DEV, max_running_requests=4, max_context=128, warm_up=False)
+    for (text, n_events, done), (prompt, n) in zip(got, jobs):
+        assert done and n_events == n + 1 and len(text.split()) == n
+        ids = server._token_request(parse(_payload(prompt, None, n))).token_ids
+        want = eng.generate([OfflineRequest(token_ids=ids, max_tokens=n)])[0].output_token_ids
+        assert text == "".join(server.tokenizer.decode(t) for t in want)
