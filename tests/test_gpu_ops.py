@@ -169,10 +169,10 @@ def test_silu_and_mul_equals_unfused():
 
 
 def _equal_but_for_last_bits(got, want, what):
-    """Equal element for element, except at most one in a thousand, and those by a rounding of the sigmoid's last place
+    """Equal element for element, except at most one in a thousand (two of a small tensor), and those by a rounding of the sigmoid's last place
     (relative 1 %; next to zero, where the sigmoid itself is a subnormal of T, 1e-6 absolute)."""
     ne = got != want
-    assert ne.float().mean().item() <= 1e-3, f"{what}: {int(ne.sum())} of {ne.numel()} elements differ"
+    assert int(ne.sum()) <= max(2, ne.numel() // 1000), f"{what}: {int(ne.sum())} of {ne.numel()} elements differ"
     g, w = got.float(), want.float()
     assert bool(((g - w).abs() <= 1e-2 * w.abs() + 1e-6).all()), f"{what}: max difference {(g - w).abs().max().item()}"
 
