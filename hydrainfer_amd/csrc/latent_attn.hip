@@ -68,8 +68,8 @@ __global__ __launch_bounds__(256) void latent_norm_cache_kernel(const typename A
 // ---------------------------------------------------------------------------------------------------------------
 // Row form: one wave per (token, head).  Keys go by in groups of 64: lane l scores key lo + l (its own row of the
 // cache against the query in LDS), the group's maximum and sum are wave reductions, then the lanes turn to the latent's
-// columns (lane l owns columns l, l + 64, ...) and add the 64 rows, each weighted by its lane's p.  Serves decode steps
-// and short portions; long portions take the tiled form below.
+// columns (lane l owns columns l, l + 64, ...) and add the 64 rows, each weighted by its lane's p.  Serves float32 runs
+// and layouts that are not 16-byte aligned; bfloat16 runs take the MFMA forms below.
 // ---------------------------------------------------------------------------------------------------------------
 constexpr int kMaxCols = HXM_MAX_LATENT / 64;
 
