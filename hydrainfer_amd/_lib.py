@@ -211,7 +211,7 @@ def lib() -> ctypes.CDLL:
 # a paged latent cache.  A library of its own, so that a model that needs only these builds only these (`make mix`).
 # ---------------------------------------------------------------------------------------------------------
 MIX_LIB_PATH = os.environ.get("HX_MIX_LIB_PATH") or os.path.join(_HERE, "lib", "libhydra_mix.so")
-HXM_ABI_VERSION = 1
+HXM_ABI_VERSION = 2
 HXM_MAX_STREAMS = 16
 HXM_MAX_LATENT = 1024
 
@@ -227,6 +227,26 @@ class hxm_latent_attn_args(ctypes.Structure):
         ("n_tokens", c_int32), ("n_seq", c_int32), ("n_heads", c_int32), ("kv_rank", c_int32), ("block_size", c_int32),
         ("window", c_int32), ("max_q_len", c_int32), ("scale", c_float), ("dtype", c_int32),
         ("max_kv_len", c_int32), ("n_splits", c_int32), ("ws_o", c_void_p), ("ws_ml", c_void_p),
+    ]
+
+
+class hxm_depth_norm_args(ctypes.Structure):
+    _fields_ = [
+        ("x_in", c_void_p), ("y", c_void_p), ("post_w", c_void_p), ("level_out", c_void_p), ("levels", c_void_p),
+        ("depth_w", c_void_p), ("x_out", c_void_p), ("next_w", c_void_p), ("h_out", c_void_p), ("rows", c_void_p),
+        ("y_stride", c_int64), ("level_stride", c_int64), ("n_out", c_int64), ("width", c_int64),
+        ("n_levels", c_int32), ("rms", c_int32), ("dtype", c_int32), ("mult", c_float), ("eps", c_float),
+    ]
+
+
+class hxm_biased_attn_args(ctypes.Structure):
+    _fields_ = [
+        ("out", c_void_p), ("q", c_void_p), ("key_cache", c_void_p), ("value_cache", c_void_p), ("slopes", c_void_p),
+        ("tok_seq", c_void_p), ("positions", c_void_p), ("block_table", c_void_p), ("cu_block_lens", c_void_p),
+        ("cache_block_stride", c_int64), ("cache_row_stride", c_int64), ("head_stride", c_int64),
+        ("n_tokens", c_int32), ("n_heads", c_int32), ("kv_heads", c_int32), ("dim", c_int32), ("vdim", c_int32),
+        ("block_size", c_int32), ("mask_kind", c_int32), ("mask_size", c_int32), ("scale", c_float), ("dtype", c_int32),
+        ("q_cu", c_void_p), ("n_seq", c_int32), ("max_q_len", c_int32),
     ]
 
 
@@ -246,6 +266,24 @@ _MIX_SIGNATURES = {
                                       c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int, c_void_p]),
     "hxm_latent_attention": (c_int, [POINTER(hxm_latent_attn_args), c_void_p]),
     "hxm_latent_attention_plan": (c_int, [POINTER(hxm_latent_attn_args), POINTER(c_int32), POINTER(c_int64)]),
+    "hxm_embed_positions": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                    c_int, c_void_p]),
+    "hxm_depth_norm": (c_int, [POINTER(hxm_depth_norm_args), c_void_p]),
+    "hxm_poly_norm": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_float, c_int64, c_int64, c_int, c_void_p]),
+    "hxm_relu_squared": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "hxm_route_softmax_topk": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int32, c_int32, c_float, c_void_p, c_void_p, c_void_p]),
+    "hxm_moe_plan": (c_int, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "hxm_grouped_linear": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int64, c_int64,
+                                   c_int32, c_int, c_void_p]),
+    "hxm_moe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64,
+                                c_int, c_void_p]),
+    "hxm_gated_recurrence": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
+                                     c_float, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32,
+                                     c_int, c_void_p]),
+    "hxm_qk_norm_cache": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+                                  c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int,
+                                  c_void_p]),
+    "hxm_biased_attention": (c_int, [POINTER(hxm_biased_attn_args), c_void_p]),
 }
 
 _mix = None

@@ -2,7 +2,11 @@
  * hydra_mix.h — C ABI of libhydra_mix.so: kernels of the sequence-mixing mechanisms that the Llama path does not have —
  * multi-stream residuals (hyper-connections) with grouped RMS norm, token shift and gated sublayer results, the tanh
  * GELU gate, and attention over a paged cache of low-rank latents (one latent row per token, shared by all heads) with a
- * sliding window.
+ * sliding window; and, for depth-averaged recurrent / attention hybrids: token + learned position embedding, layer
+ * norms around every sublayer with the residual kept in a stack of levels (depth-weighted average), the PolyNorm and
+ * squared-ReLU activations, a softmax router with a choice bias, grouped expert products over expert-major rows, a
+ * gated linear recurrence with a matrix state per head (HGRN2), and grouped-query attention over a paged key/value
+ * cache with a per-head linear distance bias and a causal, windowed or chunked mask.
  *
  * Same conventions as hydra_hip.h: raw device pointers, sizes and strides in ELEMENTS, a hipStream_t passed as void*,
  * asynchronous launches, no allocation, 0 or a negative hx_status (hydra_hip.h) as the result.  `dtype` is the hx_dtype
@@ -20,7 +24,7 @@
 extern "C" {
 #endif
 
-#define HXM_ABI_VERSION 1
+#define HXM_ABI_VERSION 2
 #define HXM_MAX_STREAMS 16
 #define HXM_MAX_LATENT 1024     /* widest latent row the attention kernels hold in registers (the MFMA tile form: 512) */
 
@@ -109,6 +113,136 @@ int hxm_latent_attention_plan(const hxm_latent_attn_args* args, int32_t* n_split
 /* Softmax attention of every query over the latents of its own sequence in the paged cache (scores and weights in
  * float).  Queries of portions and single decoded tokens may share a batch. */
 int hxm_latent_attention(const hxm_latent_attn_args* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Depth-averaged residual with layer norms (hxm_depth_norm), embeddings, activations.
+ * ------------------------------------------------------------------------------------------------------------------ */
+
+/* out[t, :] = table[ids[t], :] + pos_table[positions[t], :] in float (pos_table may be NULL).  table, pos_table: dtype.
+ * An id outside [0, vocab) or a position outside [0, n_positions) contributes zeros. */
+int hxm_embed_positions(float* out, const void* table, const void* pos_table, const void* ids, int ids_are_int64,
+                        const int32_t* positions, int64_t n_tokens, int64_t width, int64_t vocab, int64_t n_positions,
+                        int dtype, void* stream);
+
+/* One row kernel for every place where a residual meets a norm.  LN(u) = (u - mean(u)) / sqrt(var(u) + eps), var the mean
+ * squared deviation; with rms != 0: LN(u) = u / sqrt(mean(u^2) + eps).  For output row i (input row r = rows ? rows[i] : i):
+ *   x = x_in[r]
+ *   if y:         x += mult * LN(y[r]) * post_w                      (a sublayer's result enters the residual)
+ *   if level_out: level_out[r] = x                                   (the layer's own result joins the stack of levels)
+ *   if depth_w:   x = sum_{j < n_levels} depth_w[j] * levels[j][r]   (levels[j] = levels + j * level_stride; may include
+ *                                                                     the level just written)
+ *   if x_out:     x_out[i] = x
+ *   if next_w:    h_out[i] = LN(x) * next_w                          (dtype; the next sublayer's input)
+ * x_in, level_out, levels, x_out: float rows of `width` (contiguous).  y: dtype, row stride y_stride. */
+typedef struct hxm_depth_norm_args {
+  const float* x_in;
+  const void* y;
+  const float* post_w;
+  float* level_out;
+  const float* levels;
+  const float* depth_w;
+  float* x_out;
+  const float* next_w;
+  void* h_out;
+  const int32_t* rows;
+  int64_t y_stride, level_stride, n_out, width;
+  int32_t n_levels, rms, dtype;
+  float mult, eps;
+} hxm_depth_norm_args;
+int hxm_depth_norm(const hxm_depth_norm_args* args, void* stream);
+
+/* PolyNorm: out = c[0] N(z) + c[1] N(z^2) + c[2] N(z^3) + c[3], powers element by element, N(u) = u / sqrt(mean(u^2) + eps)
+ * over the row.  coef: float[4] on the device.  z, out: dtype [rows, n] with their row strides. */
+int hxm_poly_norm(void* out, int64_t out_stride, const void* z, int64_t z_stride, const float* coef, float eps, int64_t rows,
+                  int64_t n, int dtype, void* stream);
+
+/* out = max(z, 0)^2 */
+int hxm_relu_squared(void* out, int64_t out_stride, const void* z, int64_t z_stride, int64_t rows, int64_t n, int dtype,
+                     void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Mixture of experts: softmax router with a choice bias, expert-major row plan, grouped products, weighted combine.
+ * ------------------------------------------------------------------------------------------------------------------ */
+
+/* s = softmax(logits[t, 0 : n_experts]); the `top` experts with the largest s + choice_bias (NULL: s; ties: the lower
+ * expert) are chosen; weights[t, k] = s[chosen k] / (sum of the chosen s + 1e-20) * scale.  logits: float, row stride
+ * logit_stride.  weights: float [n_tokens, top], experts: int32 [n_tokens, top], in order of decreasing choice score. */
+int hxm_route_softmax_topk(const float* logits, int64_t logit_stride, const float* choice_bias, int64_t n_tokens,
+                           int32_t n_experts, int32_t top, float scale, float* weights, int32_t* experts, void* stream);
+
+/* Expert-major order of the n = n_tokens * top (token, choice) pairs: seg[e] .. seg[e + 1] are the rows of expert e
+ * (int32 [n_experts + 1]); row_of[t * top + k] = the row of pair (t, k); src[row] = t.  One launch of one workgroup. */
+int hxm_moe_plan(const int32_t* experts, int64_t n_tokens, int32_t top, int32_t n_experts, int32_t* seg, int32_t* row_of,
+                 int32_t* src, void* stream);
+
+/* Y[r, :] = act(X[src ? src[r] : r, :] . W[e]^T) for the rows r of every expert e (seg as above, n_rows = seg[n_experts]
+ * is NOT read by the host: max_rows bounds it).  X: dtype rows of k_dim with stride x_stride; W: dtype [n_experts, n_dim,
+ * k_dim]; Y: dtype [max_rows, n_dim].  act: 0 none, 1 squared ReLU.  Products accumulate in float. */
+int hxm_grouped_linear(void* y, const void* x, int64_t x_stride, const int32_t* src, const void* w, const int32_t* seg,
+                       int64_t max_rows, int32_t n_experts, int64_t n_dim, int64_t k_dim, int32_t act, int dtype, void* stream);
+
+/* out[t, :] = sum_k weights[t, k] * y[row_of[t * top + k], :] + (shared ? sigmoid(shared_gate[t * gate_stride]) * shared[t, :] : 0).
+ * y, shared, out: dtype rows of `width`; weights, shared_gate: float. */
+int hxm_moe_combine(void* out, const void* y, const int32_t* row_of, const float* weights, const void* shared,
+                    const float* shared_gate, int64_t gate_stride, int64_t n_tokens, int32_t top, int64_t width, int dtype,
+                    void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Gated linear recurrence with a matrix state per head (HGRN2): f = low + (1 - low) * sigmoid(f_pre + f_bias) per head and
+ * key channel, S <- diag(f) S + (1 - f) v^T, o = S^T silu(q_pre), then o / sqrt(mean(o^2) + eps) * norm_w over each
+ * head's value channels.  Gates, state and sums are float.
+ * q_pre, f_pre: dtype [n_tokens, heads * dim], v: dtype [n_tokens, heads * vdim] (row strides given); f_bias, low: float
+ * [heads * dim]; norm_w: float [vdim]; out: dtype [n_tokens, heads * vdim] contiguous.
+ * state: float, slot s at state + s * slot_stride, [heads, dim, vdim] contiguous within a slot.  A sequence whose portion
+ * starts at position 0 starts from a zero state (the slot is not read); the slot receives the state after the portion's
+ * last token.  q_cu: int32 [n_seq + 1]; positions: int32 [n_tokens]; slots: int32 [n_seq]. */
+int hxm_gated_recurrence(void* out, const void* q_pre, int64_t q_stride, const void* f_pre, int64_t f_stride, const void* v,
+                         int64_t v_stride, const float* f_bias, const float* low, const float* norm_w, float eps,
+                         float* state, int64_t slot_stride, const int32_t* q_cu, const int32_t* positions,
+                         const int32_t* slots, int32_t n_seq, int32_t heads, int32_t dim, int32_t vdim, int dtype,
+                         void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------------
+ * Grouped-query attention over a paged key/value cache with a linear distance bias and a mask.
+ * ------------------------------------------------------------------------------------------------------------------ */
+
+/* From a token's projection row: q = rms_norm(proj[q_off : q_off + q_size]) * q_w -> q_out [n_tokens, q_size] (one norm
+ * over the whole query projection, all heads at once; q_w NULL: no norm, a plain copy); when k_size > 0: k likewise with
+ * k_w -> the key cache, v (v_size, no norm) -> the value cache, at slot_ids[token] (slot = block * block_size + row; < 0:
+ * skipped).  A cache row holds kv_heads heads of head_stride elements; keys fill the first k_size / kv_heads of each,
+ * values the first v_size / kv_heads. */
+int hxm_qk_norm_cache(const void* proj, int64_t proj_stride, int64_t q_off, int64_t q_size, int64_t k_off, int64_t k_size,
+                      int64_t v_off, int64_t v_size, const float* q_w, const float* k_w, float eps, void* q_out,
+                      const int32_t* slot_ids, void* key_cache, void* value_cache, int64_t cache_row_stride,
+                      int64_t head_stride, int32_t kv_heads, int64_t n_tokens, int dtype, void* stream);
+
+#define HXM_MASK_CAUSAL 0   /* every j <= i */
+#define HXM_MASK_WINDOW 1   /* 0 <= i - j < mask_size */
+#define HXM_MASK_CHUNK 2    /* j <= i and floor(i / mask_size) == floor(j / mask_size), chunks counted from position 0 */
+
+typedef struct hxm_biased_attn_args {
+  void* out;                 /* dtype [n_tokens, n_heads, vdim] contiguous */
+  const void* q;             /* dtype [n_tokens, n_heads, dim] contiguous */
+  const void* key_cache;     /* dtype paged: block b at + b * cache_block_stride, row r + r * cache_row_stride, head g + g * head_stride */
+  const void* value_cache;
+  const float* slopes;       /* [n_heads] or NULL: score = q . k * scale - slopes[h] * (i - j) */
+  const int32_t* tok_seq;    /* [n_tokens] */
+  const int32_t* positions;  /* [n_tokens] */
+  const int32_t* block_table;/* flat */
+  const int32_t* cu_block_lens; /* [n_seq + 1] */
+  int64_t cache_block_stride, cache_row_stride, head_stride;
+  int32_t n_tokens, n_heads, kv_heads, dim, vdim, block_size;
+  int32_t mask_kind, mask_size;
+  float scale;
+  int32_t dtype;
+  const int32_t* q_cu;       /* [n_seq + 1]: the tile form's portions */
+  int32_t n_seq, max_q_len;
+} hxm_biased_attn_args;
+
+/* Softmax attention of every query over the keys of its own sequence that its mask lets it see (scores and weights in
+ * float).  Queries of portions and single decoded tokens may share a batch. */
+int hxm_biased_attention(const hxm_biased_attn_args* args, void* stream);
+
 
 #ifdef __cplusplus
 }
