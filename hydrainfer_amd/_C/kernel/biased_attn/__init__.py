@@ -3,7 +3,7 @@ chunked mask (csrc/biased_attn.hip, libhydra_mix.so):
     score(i, j) = q_i . k_j * scale - slopes[h] * (i - j),   softmax over the keys j that position i sees.
 Key rows (dim) and value rows (vdim) may differ in size; a cache row holds kv_heads heads of `head_size` elements and the
 keys / values fill the first dim / vdim of each.  The caches are the pool planes [n_blocks, block_size, kv_heads, head_size]
-of the block manager."""
+of the block manager; a layer with fewer heads than the pool's rows hold uses the first of each row."""
 import ctypes
 from typing import Optional
 
@@ -22,8 +22,8 @@ def _code(dtype: torch.dtype) -> int:
 
 
 def _cache_layout(cache: Tensor, kv_heads: int):
-    if cache.dim() != 4 or cache.shape[2] != kv_heads or cache.stride(3) != 1:
-        raise _lib.HydraHipError("cache planes must be [n_blocks, block_size, kv_heads, head_size] with contiguous rows")
+    if cache.dim() != 4 or cache.shape[2] < kv_heads or cache.stride(3) != 1:
+        raise _lib.HydraHipError("cache planes must be [n_blocks, block_size, >= kv_heads, head_size] with contiguous rows")
     if cache.stride(0) % cache.stride(1) or cache.stride(0) // cache.stride(1) != cache.shape[1]:
         raise _lib.HydraHipError("cache planes: a block's rows must follow each other (slot = block * block_size + row)")
     return cache.stride(0), cache.stride(1), cache.stride(2), cache.shape[1]
@@ -62,13 +62,15 @@ def qk_norm_cache(proj: Tensor, q_size: int, k_size: int, v_size: int, q_w: Opti
 
 def biased_attention(q: Tensor, key_cache: Tensor, value_cache: Tensor, vdim: int, tok_seq: Tensor, positions: Tensor,
                      q_cu: Tensor, block_table: Tensor, cu_block_lens: Tensor, scale: float,
-                     slopes: Optional[Tensor] = None, mask: str = "causal", mask_size: int = 0, max_q_len: int = 0) -> Tensor:
-    """q: [n_tokens, n_heads, dim] contiguous.  Returns [n_tokens, n_heads, vdim]."""
+                     slopes: Optional[Tensor] = None, mask: str = "causal", mask_size: int = 0, max_q_len: int = 0,
+                     kv_heads: Optional[int] = None) -> Tensor:
+    """q: [n_tokens, n_heads, dim] contiguous.  kv_heads: the key / value heads in use (the first of every cache row;
+    default: all the plane has).  Returns [n_tokens, n_heads, vdim]."""
     _lib.require_gpu(q, key_cache, value_cache, tok_seq, positions, q_cu, block_table, cu_block_lens, slopes)
     if q.dim() != 3 or not q.is_contiguous() or key_cache.dtype != q.dtype or value_cache.dtype != q.dtype:
         raise _lib.HydraHipError("biased_attention: q contiguous [n_tokens, n_heads, dim], caches of the same dtype")
     T, H, D = q.shape
-    G = key_cache.shape[2]
+    G = int(kv_heads) if kv_heads else key_cache.shape[2]
     if value_cache.stride() != key_cache.stride() or H % G:
         raise _lib.HydraHipError("biased_attention: key and value caches of one layout; heads a multiple of kv heads")
     bstride, rstride, hstride, bs = _cache_layout(key_cache, G)

@@ -145,3 +145,15 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], laye
         if layers_out is not None:
             layers_out.append(x)
     return layer_norm(x, W["final.norm"], eps) @ W["head"].T
+
+
+def greedy(cfg, weights, prompt: List[int], n_new: int):
+    """(tokens generated greedily, top-1 margin of every step)."""
+    toks, out, margins = list(prompt), [], []
+    for _ in range(n_new):
+        last = forward(cfg, weights, toks)[-1]
+        top = torch.topk(last, 2).values
+        out.append(int(torch.argmax(last)))
+        margins.append(float(top[0] - top[1]))
+        toks.append(out[-1])
+    return out, margins
