@@ -63,9 +63,12 @@ def qk_norm_cache(proj: Tensor, q_size: int, k_size: int, v_size: int, q_w: Opti
 def biased_attention(q: Tensor, key_cache: Tensor, value_cache: Tensor, vdim: int, tok_seq: Tensor, positions: Tensor,
                      q_cu: Tensor, block_table: Tensor, cu_block_lens: Tensor, scale: float,
                      slopes: Optional[Tensor] = None, mask: str = "causal", mask_size: int = 0, max_q_len: int = 0,
-                     kv_heads: Optional[int] = None) -> Tensor:
+                     kv_heads: Optional[int] = None, max_kv_len: int = 0, form: str = "auto") -> Tensor:
     """q: [n_tokens, n_heads, dim] contiguous.  kv_heads: the key / value heads in use (the first of every cache row;
-    default: all the plane has).  Returns [n_tokens, n_heads, vdim]."""
+    default: all the plane has).  max_q_len: the longest portion of the batch; max_kv_len: the most keys a sequence holds —
+    with few rows in the launch (decode steps) the keys of every tile are dealt to several waves.  form: "auto" (bfloat16
+    with sizes that are multiples of 8: the MFMA tile form) or "rows" (one wave per token and head, any dtype and size).
+    Returns [n_tokens, n_heads, vdim]."""
     _lib.require_gpu(q, key_cache, value_cache, tok_seq, positions, q_cu, block_table, cu_block_lens, slopes)
     if q.dim() != 3 or not q.is_contiguous() or key_cache.dtype != q.dtype or value_cache.dtype != q.dtype:
         raise _lib.HydraHipError("biased_attention: q contiguous [n_tokens, n_heads, dim], caches of the same dtype")
@@ -95,5 +98,18 @@ def biased_attention(q: Tensor, key_cache: Tensor, value_cache: Tensor, vdim: in
     a.n_tokens, a.n_heads, a.kv_heads, a.dim, a.vdim = T, H, G, D, int(vdim)
     a.mask_kind, a.mask_size, a.scale, a.dtype = MASK_KINDS[mask], int(mask_size), float(scale), _code(q.dtype)
     a.n_seq, a.max_q_len = n_seq, int(max_q_len)
+    a.form, a.n_splits, a.ws_o, a.ws_ml = {"auto": 0, "rows": 1}[form], 1, None, None
+    if form == "auto" and q.dtype == torch.bfloat16 and max_q_len > 0 and max_kv_len > 0 and D % 8 == 0 and vdim % 8 == 0 \
+            and D <= 256 and vdim <= 256:
+        # key splits: enough waves to fill the chip when the launch has few row tiles, at least two 32-key chunks a split
+        tiles = n_seq * G * ((max_q_len * (H // G) + 15) // 16)
+        reach = max_kv_len
+        if mask != "causal":
+            reach = min(reach, mask_size + (max_q_len if mask == "window" else 0))
+        ns = min((2048 + tiles - 1) // tiles, ((reach + 31) // 32) // 2, 64)
+        if ns > 1:
+            v16 = (vdim + 15) // 16 * 16
+            ws = torch.empty(tiles * ns * 16 * (v16 + 2), dtype=torch.float32, device=q.device)
+            a.n_splits, a.ws_o, a.ws_ml = ns, ws.data_ptr(), ws.data_ptr() + 4 * tiles * ns * 16 * v16
     _lib.mix_check(_lib.mix_lib().hxm_biased_attention(ctypes.byref(a), _lib.current_stream()), "biased_attention")
     return out

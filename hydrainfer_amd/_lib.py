@@ -246,7 +246,8 @@ class hxm_biased_attn_args(ctypes.Structure):
         ("cache_block_stride", c_int64), ("cache_row_stride", c_int64), ("head_stride", c_int64),
         ("n_tokens", c_int32), ("n_heads", c_int32), ("kv_heads", c_int32), ("dim", c_int32), ("vdim", c_int32),
         ("block_size", c_int32), ("mask_kind", c_int32), ("mask_size", c_int32), ("scale", c_float), ("dtype", c_int32),
-        ("q_cu", c_void_p), ("n_seq", c_int32), ("max_q_len", c_int32),
+        ("q_cu", c_void_p), ("n_seq", c_int32), ("max_q_len", c_int32), ("form", c_int32), ("n_splits", c_int32),
+        ("ws_o", c_void_p), ("ws_ml", c_void_p),
     ]
 
 

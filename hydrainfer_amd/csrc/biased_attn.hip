@@ -4,7 +4,7 @@
 // kernel in front of it: one RMS norm over a token's whole query projection and one over its whole key projection
 // (all heads at once), keys and values straight into the cache.
 #include <cfloat>
-#include "hx_common.h"
+#include "attn_common.h"
 #include "../../include/hydra_mix.h"
 
 namespace hxm {
@@ -159,6 +159,264 @@ __global__ __launch_bounds__(256) void biased_attn_rows_kernel(hxm_biased_attn_a
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Tile form (bfloat16): one wave per 16 rows, a row being a (token, query head) pair of ONE sequence's portion and ONE
+// key/value head, the group's query heads fastest — the heads of a decoded token that share a key head, or a few tokens
+// times those heads.  All rows of a tile read the same keys, which go by in chunks of 32: S = Q K^T and O += P V are
+// 16x16x32 MFMAs.  Key rows come straight from the paged cache into the B operands of S (a lane's 16 bytes are 8
+// consecutive columns of one key's row); value rows are written to the wave's LDS as they come (row-major image of the
+// chunk) and return through the transposing LDS read as B operands of the second product; P goes through LDS from the
+// accumulator layout to the A layout.  Bias and mask are applied to the float scores, row by row.  With n_splits > 1 the
+// key range of a tile is dealt to several waves whose partial results a second kernel merges.  No workgroup barriers.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kPStride = 36;       // u16 per row of P in LDS: 32 slots + 4
+
+template <int KK>                  // ceil(max(dim, vdim) / 32): 1, 2, 4, 8
+__global__ __launch_bounds__(256) void biased_attn_tile_kernel(hxm_biased_attn_args a, int tiles_per_seq, int waves_per_block) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (wave >= waves_per_block) return;
+  const int n_splits = a.n_splits > 1 ? a.n_splits : 1;
+  const int G = a.kv_heads, R = a.n_heads / a.kv_heads, D = a.dim, V = a.vdim;
+  const int64_t witem = (int64_t)blockIdx.x * waves_per_block + wave;      // (sequence, kv head, row tile, key split), splits fastest
+  if (witem >= (int64_t)a.n_seq * G * tiles_per_seq * n_splits) return;
+  const int64_t item = witem / n_splits;
+  const int split = (int)(witem % n_splits);
+  const int tile = (int)(item % tiles_per_seq);
+  const int kvh = (int)((item / tiles_per_seq) % G);
+  const int b = (int)(item / ((int64_t)tiles_per_seq * G));
+  const int q0 = a.q_cu[b];
+  const int n_rows = (a.q_cu[b + 1] - q0) * R;
+  if (tile * 16 >= n_rows) return;
+  const int g = lane >> 4, c = lane & 15;
+  const int RS = 2 * (KK * 32) + 32;      // bytes per row of the value image (a key's columns, padded)
+  char* img = reinterpret_cast<char*>(lds) + (size_t)wave * (32 * RS + 16 * kPStride * 2);
+  u16* pl = reinterpret_cast<u16*>(img + 32 * RS);
+  const u16* kc = (const u16*)a.key_cache + (int64_t)kvh * a.head_stride;
+  const u16* vc = (const u16*)a.value_cache + (int64_t)kvh * a.head_stride;
+  const int32_t* table = a.block_table + a.cu_block_lens[b];
+  const u16x8 zero8 = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+
+  // the queries: lane (g, c) holds row c, columns 32 kk + 8 g .. + 7
+  const int last_row = min(tile * 16 + 15, n_rows - 1);
+  u16x8 qf[KK];
+  {
+    const int r = min(tile * 16 + c, n_rows - 1);
+    const u16* qg = (const u16*)a.q + ((int64_t)(q0 + r / R) * a.n_heads + kvh * R + r % R) * D;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int col = 32 * kk + 8 * g;
+      qf[kk] = col < D ? *reinterpret_cast<const u16x8*>(qg + col) : zero8;
+    }
+  }
+  // the rows this lane holds of S and O: 4 g + i
+  int pos[4], lo[4];
+  float slope[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 16 + 4 * g + i;
+    if (r < n_rows) {
+      pos[i] = a.positions[q0 + r / R];
+      lo[i] = first_visible(pos[i], a.mask_kind, a.mask_size);
+      slope[i] = a.slopes ? a.slopes[kvh * R + r % R] : 0.f;
+    } else {
+      pos[i] = -1;      // sees nothing
+      lo[i] = 0;
+      slope[i] = 0.f;
+    }
+  }
+  // the keys any row of the tile sees
+  int k_min, k_max;
+  {
+    const int r = min(tile * 16 + c, last_row);
+    const int pr = a.positions[q0 + r / R];
+    k_max = pr;
+    k_min = first_visible(pr, a.mask_kind, a.mask_size);
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) {
+      k_max = max(k_max, __shfl_xor(k_max, off, 64));
+      k_min = min(k_min, __shfl_xor(k_min, off, 64));
+    }
+  }
+  float m[4], l[4];
+  f32x4 acc[KK * 2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { m[i] = -1.0e30f; l[i] = 0.f; }
+#pragma unroll
+  for (int n = 0; n < KK * 2; ++n) acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+  int k_begin = k_min, k_end = k_max;
+  if (n_splits > 1) {
+    const int chunks = (k_max - k_min + 32) / 32;
+    const int per = (chunks + n_splits - 1) / n_splits;
+    k_begin = k_min + split * per * 32;
+    k_end = min(k_max, k_begin + per * 32 - 1);
+  }
+  const int bs = a.block_size;
+  const int bshift = (bs & (bs - 1)) == 0 ? __ffs(bs) - 1 : -1;
+  for (int key0 = k_begin; key0 <= k_end; key0 += 32) {
+    // half a chunk's rows, this lane's part: key 16 s + c, columns 32 kk + 8 g .. + 7
+    u16x8 kf[2][KK], vf[2][KK];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int key = min(key0 + 16 * s + c, k_max);        // (a key past the last one repeats it; masked below)
+      const int page = bshift >= 0 ? key >> bshift : key / bs;
+      const int64_t off = (int64_t)table[page] * a.cache_block_stride + (int64_t)(key - page * bs) * a.cache_row_stride;
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        const int col = 32 * kk + 8 * g;
+        kf[s][kk] = col < D ? *reinterpret_cast<const u16x8*>(kc + off + col) : zero8;
+        vf[s][kk] = col < V ? *reinterpret_cast<const u16x8*>(vc + off + col) : zero8;
+      }
+    }
+    f32x4 sc[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      sc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) {
+        sc[s] = Mfma<BF16>::mma(qf[kk], kf[s][kk], sc[s]);
+        *reinterpret_cast<u16x8*>(img + (16 * s + c) * RS + (32 * kk + 8 * g) * 2) = vf[s][kk];
+      }
+    }
+    // softmax of the rows 4 g + i over this chunk (sc[s][i] is key key0 + 16 s + c)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float p[2];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        const int key = key0 + 16 * s + c;
+        const bool seen = key >= lo[i] && key <= pos[i];
+        p[s] = seen ? sc[s][i] * a.scale - slope[i] * (float)(pos[i] - key) : -INFINITY;
+        mx = fmaxf(mx, p[s]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
+      const float m_new = fmaxf(m[i], mx);
+      const float corr = __expf(m[i] - m_new);
+      p[0] = __expf(p[0] - m_new);       // exp(-inf) = 0 for a key the row does not see
+      p[1] = __expf(p[1] - m_new);
+      float ps = p[0] + p[1];
+      ps += __shfl_xor(ps, 1, 64);
+      ps += __shfl_xor(ps, 2, 64);
+      ps += __shfl_xor(ps, 4, 64);
+      ps += __shfl_xor(ps, 8, 64);
+      l[i] = l[i] * corr + ps;
+      m[i] = m_new;
+#pragma unroll
+      for (int n = 0; n < KK * 2; ++n) acc[n][i] *= corr;
+      // key 16 s + c sits in slot 8 (c / 4) + c % 4 + 4 s of its row: the order the transposing read delivers the keys in
+      pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3)] = BF16::from_float(p[0]);
+      pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3) + 4] = BF16::from_float(p[1]);
+    }
+    wave_lds_sync();
+    // O += P V: A = P[row c][slots 8 g ..], B = the image's column 16 n + c at the keys of those slots
+    u16x8 pf;
+    {
+      const u16x4 x0 = *reinterpret_cast<const u16x4*>(pl + c * kPStride + 8 * g);
+      const u16x4 x1 = *reinterpret_cast<const u16x4*>(pl + c * kPStride + 8 * g + 4);
+      pf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+    }
+    const char* vrd = img + (4 * g + (c >> 2)) * RS + (c & 3) * 8;
+#pragma unroll
+    for (int n = 0; n < KK * 2; ++n) {
+      const u16x4 x0 = lds_tr_read(vrd + n * 32);
+      const u16x4 x1 = lds_tr_read(vrd + 16 * RS + n * 32);
+      const u16x8 vv = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+      acc[n] = Mfma<BF16>::mma(pf, vv, acc[n]);
+    }
+    wave_lds_sync();      // the reads are done before the next chunk is written
+  }
+  const int V16 = (V + 15) / 16 * 16;
+  if (n_splits > 1) {
+    // unnormalised partial result of this split: ws_o [item][split][16 rows][V16], ws_ml [item][split][16 rows][m, l]
+    float* wo = a.ws_o + ((size_t)witem * 16) * V16;
+    float* wml = a.ws_ml + (size_t)witem * 32;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 4 * g + i;
+      if (c == 0) {
+        wml[2 * row] = m[i];
+        wml[2 * row + 1] = l[i];
+      }
+#pragma unroll
+      for (int n = 0; n < KK * 2; ++n) {
+        const int col = 16 * n + c;
+        if (col < V16) wo[(size_t)row * V16 + col] = acc[n][i];
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 16 + 4 * g + i;
+    if (r >= n_rows) continue;
+    const float inv = 1.0f / l[i];
+    u16* og = (u16*)a.out + ((int64_t)(q0 + r / R) * a.n_heads + kvh * R + r % R) * V;
+#pragma unroll
+    for (int n = 0; n < KK * 2; ++n) {
+      const int col = 16 * n + c;
+      if (col < V) og[col] = BF16::from_float(acc[n][i] * inv);
+    }
+  }
+}
+
+// the splits of a (sequence, kv head, row tile) merged: out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M)
+__global__ __launch_bounds__(256) void biased_attn_combine_kernel(hxm_biased_attn_args a, int tiles_per_seq) {
+  const int64_t item = blockIdx.x;
+  const int G = a.kv_heads, R = a.n_heads / a.kv_heads, V = a.vdim, V16 = (V + 15) / 16 * 16, NS = a.n_splits;
+  const int tile = (int)(item % tiles_per_seq);
+  const int kvh = (int)((item / tiles_per_seq) % G);
+  const int b = (int)(item / ((int64_t)tiles_per_seq * G));
+  const int q0 = a.q_cu[b];
+  const int n_rows = (a.q_cu[b + 1] - q0) * R;
+  if (tile * 16 >= n_rows) return;
+  __shared__ float wgt[16][65];      // [row][split] weight e^(m_s - M) / L (NS <= 64)
+  if (threadIdx.x < 16) {
+    const int row = threadIdx.x;
+    const float* wml = a.ws_ml + (size_t)item * NS * 32;
+    float M = -1.0e30f;
+    for (int s = 0; s < NS; ++s) M = fmaxf(M, wml[s * 32 + 2 * row]);
+    float L = 0.f;
+    for (int s = 0; s < NS; ++s) L += wml[s * 32 + 2 * row + 1] * __expf(wml[s * 32 + 2 * row] - M);
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    for (int s = 0; s < NS; ++s) wgt[row][s] = __expf(wml[s * 32 + 2 * row] - M) * inv;
+  }
+  __syncthreads();
+  const float* wo = a.ws_o + (size_t)item * NS * 16 * V16;
+  for (int e = threadIdx.x; e < 16 * V; e += 256) {
+    const int row = e / V, col = e % V;
+    const int r = tile * 16 + row;
+    if (r >= n_rows) continue;
+    float v = 0.f;
+    for (int s = 0; s < NS; ++s) v += wo[((size_t)s * 16 + row) * V16 + col] * wgt[row][s];
+    ((u16*)a.out)[((int64_t)(q0 + r / R) * a.n_heads + kvh * R + r % R) * V + col] = BF16::from_float(v);
+  }
+}
+
+template <int KK>
+int launch_tile(const hxm_biased_attn_args& a, hipStream_t s) {
+  const size_t per_wave = (size_t)32 * (2 * (KK * 32) + 32) + 16 * kPStride * 2;
+  int waves = 4;
+  while (waves > 1 && per_wave * waves > 64 * 1024) waves >>= 1;
+  const int R = a.n_heads / a.kv_heads;
+  const int tiles_per_seq = (int)(((int64_t)a.max_q_len * R + 15) / 16);
+  const int n_splits = a.n_splits > 1 ? a.n_splits : 1;
+  const int64_t items = (int64_t)a.n_seq * a.kv_heads * tiles_per_seq;
+  const dim3 grid((unsigned)((items * n_splits + waves - 1) / waves));
+  biased_attn_tile_kernel<KK><<<grid, dim3(64 * waves), per_wave * waves, s>>>(a, tiles_per_seq, waves);
+  if (n_splits > 1) biased_attn_combine_kernel<<<dim3((unsigned)items), dim3(256), 0, s>>>(a, tiles_per_seq);
+  return hxm::check_launch();
+}
+
+bool tile_form_serves(const hxm_biased_attn_args& a) {
+  const bool aligned = a.dim % 8 == 0 && a.vdim % 8 == 0 && a.head_stride % 8 == 0 && a.cache_row_stride % 8 == 0 &&
+                       a.cache_block_stride % 8 == 0 && aligned16(a.key_cache) && aligned16(a.value_cache) && aligned16(a.q);
+  return a.dtype == HX_BF16 && aligned && a.dim <= 256 && a.vdim <= 256 && a.q_cu && a.n_seq > 0 && a.max_q_len > 0 && a.form != 1;
+}
+
 }  // namespace
 
 extern "C" int hxm_qk_norm_cache(const void* proj, int64_t proj_stride, int64_t q_off, int64_t q_size, int64_t k_off,
@@ -203,6 +461,14 @@ extern "C" int hxm_biased_attention(const hxm_biased_attn_args* args, void* stre
   if (!a.out || !a.q || !a.key_cache || !a.value_cache || !a.tok_seq || !a.positions || !a.block_table || !a.cu_block_lens) return HX_ERR_NULL;
   if (a.dim > a.head_stride || a.vdim > a.head_stride) return HX_ERR_STRIDE;
   hipStream_t s = (hipStream_t)stream;
+  if (a.n_splits > 1 && (a.n_splits > 64 || !a.ws_o || !a.ws_ml || !tile_form_serves(a))) return HX_ERR_WORKSPACE;
+  if (tile_form_serves(a)) {
+    const int kk = ((a.dim > a.vdim ? a.dim : a.vdim) + 31) / 32;
+    if (kk <= 1) return launch_tile<1>(a, s);
+    if (kk <= 2) return launch_tile<2>(a, s);
+    if (kk <= 4) return launch_tile<4>(a, s);
+    return launch_tile<8>(a, s);
+  }
   const int64_t items = (int64_t)a.n_tokens * a.n_heads;
   const size_t lds = 4 * ((size_t)a.dim + 64) * sizeof(float);
   if (lds > 64 * 1024) return HX_ERR_SHAPE;

@@ -367,7 +367,7 @@ class KezolixForCausalLM:
             q = qk_norm_cache(proj, H * D, 0, 0, w.q_norm, None, sh.norm_eps, G)
         o = biased_attention(q.view(T, H, D), kc, vc, V, seq.tok_seq, position_ids, ap.q_cu_seq_lens, ap.block_tables,
                              ap.cu_blocks_lens, m.scale, w.slopes, "chunk" if m.chunk else "causal", m.chunk or 0,
-                             max_q_len=ap.q_max_seq_len, kv_heads=G)
+                             max_q_len=ap.q_max_seq_len, kv_heads=G, max_kv_len=ap.kv_max_seq_len)
         return torch.matmul(o.view(T, H * V), w.o.t())
 
     def _recurrence(self, i: int, h: Tensor, position_ids: Tensor, params, seq: SequenceState) -> Tensor:

@@ -1,6 +1,6 @@
-"""`bench.py --design tetepel`: prefill and decode throughput of the Tetepel design at sizes that resemble a real model's
-layers (random weights, a few layers), beside the Llama decoder at equal width / feed-forward / heads, and a table of
-the design's own kernels against the Llama path's like kernels, each as a fraction of its roofline (HBM bytes or MFMA
+"""`bench.py --design tetepel|kezolix`: prefill and decode throughput of a model design at sizes that resemble a real
+model's layers (random weights, a few layers), beside the Llama decoder at equal width / feed-forward / heads, and a table
+of the design's own kernels against the Llama path's like kernels, each as a fraction of its roofline (HBM bytes or MFMA
 flops, algorithmic counts).  Both models run their eager step (no captured graph / launch plan) on hand-built batches."""
 import math
 import time
@@ -28,6 +28,21 @@ def _tetepel(size: dict, dtype, dev):
     return TetepelForCausalLM.random_init(shape, dtype, dev, seed=0)
 
 
+def _kezolix(size: dict, dtype, dev):
+    """Four layers: recurrent + dense, attention + experts, recurrent + experts, attention on the second layer's keys +
+    experts.  Attention as wide as the Llama decoder's (a quarter of the heads carry keys), chunks of 512; the recurrent
+    layers keep a 128 x 128 state per head; 16 experts of a quarter of the dense inner size, four a token, and a shared one."""
+    from hydrainfer_amd.model.kezolix import FeedForwardSpec, KezolixForCausalLM, KezolixLayer, KezolixShape, MixerSpec
+    H, D, ff = size["heads"], size["dim"], size["ff"]
+    att = lambda kv_from: MixerSpec("attention", H, D, D, H // 4, 1.0 / math.sqrt(D), 512, kv_from)
+    rec = MixerSpec("hgrn2", H, D, D)
+    moe = FeedForwardSpec("moe", ff // 4 // 32 * 32, 16, 4, 1.0, ff // 4 // 32 * 32)
+    layers = [KezolixLayer(rec, FeedForwardSpec("dense", ff)), KezolixLayer(att(None), moe), KezolixLayer(rec, moe),
+              KezolixLayer(att(1), moe)][:size["layers"]]
+    shape = KezolixShape(VOCAB, size["width"], layers, max_position_embeddings=8192, norm_eps=1e-5, residual_mult=0.5)
+    return KezolixForCausalLM.random_init(shape, dtype, dev, seed=0)
+
+
 def _llama(size: dict, dtype, dev):
     from hydrainfer_amd.model.llama import LlamaForCausalLM, LlamaShape
     shape = LlamaShape(size["width"], size["ff"], size["layers"], size["heads"], size["heads"], size["dim"], VOCAB)
@@ -45,17 +60,19 @@ def _batch(model, n_seqs: int, q_len: int, kv_len: int, dtype, dev):
     for s in range(n_seqs):
         table = list(range(s * nb, (s + 1) * nb))
         b.add_request(q_len, kv_len, [table[p // bs] * bs + p % bs for p in range(kv_len - q_len, kv_len)], table)
-    latent = hasattr(model, "cache_spec")
-    for _ in range(sh.num_hidden_layers):
-        k = torch.randn((n_seqs * nb, bs, sh.num_key_value_heads, sh.head_dim), device=dev).to(dtype)
-        b.add_kv_cache(KVCache(k, k if latent else torch.randn_like(k)))
+    spec = model.cache_spec() if hasattr(model, "cache_spec") else {
+        "n_layers": sh.num_hidden_layers, "n_tokens": 2, "n_heads": sh.num_key_value_heads, "head_size": sh.head_dim}
+    for _ in range(spec["n_layers"]):
+        k = torch.randn((n_seqs * nb, bs, spec["n_heads"], spec["head_size"]), device=dev).to(dtype)
+        b.add_kv_cache(KVCache(k, k if spec["n_tokens"] == 1 else torch.randn_like(k)))
     ap = b.build_attention_parameters()
     pos = torch.arange(kv_len - q_len, kv_len, dtype=torch.int32, device=dev).repeat(n_seqs)
     sel = torch.arange(q_len - 1, n_seqs * q_len, q_len, device=dev)
     params = LanguageModelParameters(ap, q_len == 1, sel)
-    if latent:
+    sspec = model.state_spec() if hasattr(model, "state_spec") else None
+    if sspec is not None:
         from hydrainfer_amd._C.kernel.stream_ops import SequenceState
-        state = torch.zeros((n_seqs, sh.num_hidden_layers, sh.hidden_size), dtype=torch.float32, device=dev)
+        state = torch.zeros((n_seqs, sspec["rows"], sspec["width"]), dtype=torch.float32, device=dev)
         params.sequence_state = SequenceState(state, torch.arange(n_seqs, dtype=torch.int32, device=dev),
                                               torch.arange(n_seqs, dtype=torch.int32, device=dev).repeat_interleave(q_len))
     ids = torch.randint(0, VOCAB, (n_seqs * q_len,), device=dev, dtype=torch.int32)
@@ -106,10 +123,10 @@ def _row(name, us, nbytes=None, flops=None):
     return r
 
 
-def throughput(size_name: str, dtype, dev, prefill=(4, 1024), decode=(32, 1024)) -> dict:
+def throughput(size_name: str, dtype, dev, prefill=(4, 1024), decode=(32, 1024), design: str = "tetepel") -> dict:
     size = SIZES[size_name]
     out = {}
-    for name, make in (("tetepel", _tetepel), ("llama", _llama)):
+    for name, make in ((design, {"tetepel": _tetepel, "kezolix": _kezolix}[design]), ("llama", _llama)):
         model = make(size, dtype, dev)
         if name == "llama":
             model.prepare_decode(max_rows=decode[0])
@@ -207,11 +224,156 @@ def kernel_table(size_name: str, dtype, dev, T: int = 4096, n_seqs: int = 4, B: 
     return rows
 
 
-def run(dtype, dev, sizes=("w2048", "w4096")) -> dict:
+def _llama_rows(size_name: str, dtype, dev, T: int, n_seqs: int, B: int, ctx: int) -> List[dict]:
+    """The Llama path's kernels that the designs' kernels are set beside, at the same sizes."""
+    from hydrainfer_amd._C.kernel.activation import silu_and_mul
+    from hydrainfer_amd._C.kernel.flash_attn import mha_varlen_fwd
+    from hydrainfer_amd._C.kernel.norm import add_rms_norm
+    from hydrainfer_amd._C.kernel.position_embedding import rope_set_kv_cache
+    sz = SIZES[size_name]
+    W, ff, H, D = sz["width"], sz["ff"], sz["heads"], sz["dim"]
+    e = 2
+    rnd = lambda *s: torch.randn(s, device=dev).to(dtype)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev) if not torch.is_tensor(v) else v.to(torch.int32).to(dev)
+    rows = []
+    q_len = T // n_seqs
+    nb, nbd = (q_len + 15) // 16, (ctx + 15) // 16
+    q_cu = i32(list(range(0, T + 1, q_len)))
+    pos = torch.arange(q_len, dtype=torch.int32, device=dev).repeat(n_seqs)
+    table, cu_b = i32(torch.randperm(n_seqs * nb)), i32(list(range(0, n_seqs * nb + 1, nb)))
+    slots = i32([int(table[s * nb + p // 16]) * 16 + p % 16 for s in range(n_seqs) for p in range(q_len)])
+    res, xx, out, w16, gu = rnd(T, W), rnd(T, W), rnd(T, W), rnd(W), rnd(T, 2 * ff)
+    us = _time_graph(lambda: add_rms_norm(out, res, xx, w16, 1e-6), dev)
+    rows.append(_row("add_rms_norm (residual add + norm)", us, 4 * T * W * e))
+    us = _time_graph(lambda: silu_and_mul(gu[:, :ff], gu[:, ff:]), dev)
+    rows.append(_row("silu_and_mul", us, 3 * T * ff * e))
+    q, k, v = rnd(T, H, D), rnd(T, H, D), rnd(T, H, D)
+    kc, vc = rnd(n_seqs * nb, 16, H, D), rnd(n_seqs * nb, 16, H, D)
+    cos_sin = rnd(max(q_len, ctx), 2, D // 2)
+    us = _time_graph(lambda: rope_set_kv_cache(q, k, v, pos, cos_sin, D, slots, kc, vc), dev)
+    rows.append(_row("rope_set_kv_cache (rotary + cache append)", us, (2 * 2 * T * H * D + 2 * T * H * D) * e))
+    o = torch.empty_like(q)
+    us = _time_graph(lambda: mha_varlen_fwd(o, q, kc, vc, q_cu, q_cu, table, cu_b, None, q_len, q_len, 1 / math.sqrt(D), 0, -1, 0, 0), dev, launches=4)
+    rows.append(_row(f"mha_varlen_fwd, prefill {n_seqs} x {q_len} (causal, head_dim {D})", us,
+                     flops=4 * H * D * n_seqs * sum(i + 1 for i in range(q_len))))
+    table_d, cu_bd = i32(torch.randperm(B * nbd)), i32(list(range(0, B * nbd + 1, nbd)))
+    kcd, vcd = rnd(B * nbd, 16, H, D), rnd(B * nbd, 16, H, D)
+    qd2, od2 = rnd(B, H, D), rnd(B, H, D)
+    qcud, cu_kd = i32(list(range(B + 1))), i32(list(range(0, B * ctx + 1, ctx)))
+    us = _time_graph(lambda: mha_varlen_fwd(od2, qd2, kcd, vcd, qcud, cu_kd, table_d, cu_bd, None, 1, ctx, 1 / math.sqrt(D), 0, -1, 0, 0), dev)
+    rows.append(_row(f"mha_varlen_fwd, decode {B} x {ctx} keys", us, 2 * B * ctx * H * D * e + 2 * B * H * D * e))
+    return rows
+
+
+def kezolix_kernel_table(size_name: str, dtype, dev, T: int = 4096, n_seqs: int = 4, B: int = 32, ctx: int = 2048) -> dict:
+    """Every kernel of the Kezolix design at a prefill batch of T tokens (n_seqs portions) — attention and recurrence also
+    at a decode batch of B sequences — and the Llama path's like kernels at the same sizes."""
+    from hydrainfer_amd._C.kernel import biased_attn as ba, depth_ops as do, moe_mix as mm
+    from hydrainfer_amd._C.kernel.recurrence import gated_recurrence
+    from hydrainfer_amd._C.kernel.stream_ops import SequenceState
+    sz = SIZES[size_name]
+    W, ff, H, D = sz["width"], sz["ff"], sz["heads"], sz["dim"]
+    G, V, chunk, E, top, n_lv = H // 4, D, 512, 16, 4, 5
+    eff = ff // 4 // 32 * 32
+    e = 2
+    rnd = lambda *s: torch.randn(s, device=dev).to(dtype)
+    f32 = lambda *s: torch.randn(s, device=dev)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev) if not torch.is_tensor(v) else v.to(torch.int32).to(dev)
+    rows: Dict[str, List[dict]] = {"kezolix": [], "llama": []}
+    add = lambda *a, **k: rows["kezolix"].append(_row(*a, **k))
+    q_len = T // n_seqs
+    q_cu = i32(list(range(0, T + 1, q_len)))
+    pos = torch.arange(q_len, dtype=torch.int32, device=dev).repeat(n_seqs)
+    tok_seq = torch.arange(n_seqs, dtype=torch.int32, device=dev).repeat_interleave(q_len)
+    x, y, w1, w2 = f32(T, W), rnd(T, W), f32(W), f32(W)
+    xo, levels, dw = torch.empty_like(x), f32(n_lv, T, W), f32(n_lv)
+    us = _time_graph(lambda: do.depth_norm(x, dtype, 1e-5, y=y, post_w=w1, mult=0.5, x_out=xo, next_w=w2), dev)
+    add("depth_norm, mid-layer (norm of y into the residual + next norm)", us, T * W * (8 + 2 * e))
+    us = _time_graph(lambda: do.depth_norm(x, dtype, 1e-5, y=y, post_w=w1, mult=0.5, level_out=levels[n_lv - 1], levels=levels,
+                                           depth_w=dw, x_out=xo, next_w=w2), dev)
+    add(f"depth_norm, layer end (+ level written, average of {n_lv} levels)", us, T * W * (4 * (n_lv + 2) + 2 * e))
+    z, coef = rnd(T, ff), f32(4)
+    us = _time_graph(lambda: do.poly_norm(z, coef, 1e-5), dev)
+    add("poly_norm", us, 2 * T * ff * e)
+    # recurrence: prefill portions from position 0, then one token for B sequences
+    proj = rnd(T, 3 * H * D)
+    fb, low, nw = f32(H * D), torch.rand(H * D, device=dev), f32(V)
+    state = torch.zeros((max(n_seqs, B), 1, H * D * V), device=dev)
+    seq = SequenceState(state, i32(list(range(n_seqs))), tok_seq)
+    us = _time_graph(lambda: gated_recurrence(proj[:, :H * D], proj[:, H * D:2 * H * D], proj[:, 2 * H * D:], fb, low, nw, 1e-5, seq, 0,
+                                              q_cu, pos, H, D, V), dev, launches=2)
+    add(f"gated_recurrence, prefill {n_seqs} x {q_len} ({H} heads, state {D} x {V})", us, flops=6 * T * H * D * V)
+    posd, qcud = i32([ctx - 1] * B), i32(list(range(B + 1)))
+    seqd = SequenceState(state, i32(list(range(B))), i32(list(range(B))))
+    us = _time_graph(lambda: gated_recurrence(proj[:B, :H * D], proj[:B, H * D:2 * H * D], proj[:B, 2 * H * D:], fb, low, nw, 1e-5, seqd,
+                                              0, qcud, posd, H, D, V), dev)
+    add(f"gated_recurrence, decode {B} sequences (state read and written)", us, 2 * B * H * D * V * 4)
+    # attention
+    nb, nbd = (q_len + 15) // 16, (ctx + 15) // 16
+    kc, vc = rnd(n_seqs * nb, 16, G, D), rnd(n_seqs * nb, 16, G, D)
+    table, cu_b = i32(torch.randperm(n_seqs * nb)), i32(list(range(0, n_seqs * nb + 1, nb)))
+    slots = i32([int(table[s * nb + p // 16]) * 16 + p % 16 for s in range(n_seqs) for p in range(q_len)])
+    qkv, qw, kw = rnd(T, (H + 2 * G) * D), f32(H * D), f32(G * D)
+    us = _time_graph(lambda: ba.qk_norm_cache(qkv, H * D, G * D, G * V, qw, kw, 1e-5, G, slots, kc, vc), dev)
+    add("qk_norm_cache (two norms + cache append)", us, T * (2 * H * D + 2 * G * D + 2 * G * V) * e)
+    q = rnd(T, H, D)
+    slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)], device=dev)
+    seen = n_seqs * sum(i % chunk + 1 for i in range(q_len))
+    us = _time_graph(lambda: ba.biased_attention(q, kc, vc, V, tok_seq, pos, q_cu, table, cu_b, 1 / math.sqrt(D), slopes, "chunk", chunk,
+                                                 max_q_len=q_len), dev, launches=2)
+    add(f"biased_attention, prefill {n_seqs} x {q_len} (chunks of {chunk}, head_dim {D})", us, flops=2 * H * (D + V) * seen)
+    kcd, vcd = rnd(B * nbd, 16, G, D), rnd(B * nbd, 16, G, D)
+    table_d, cu_bd = i32(torch.randperm(B * nbd)), i32(list(range(0, B * nbd + 1, nbd)))
+    qd, seq_ids = rnd(B, H, D), i32(list(range(B)))
+    keys = (ctx - 1) % chunk + 1
+    us = _time_graph(lambda: ba.biased_attention(qd, kcd, vcd, V, seq_ids, posd, qcud, table_d, cu_bd, 1 / math.sqrt(D), slopes, "chunk",
+                                                 chunk, max_q_len=1), dev)
+    add(f"biased_attention, decode {B} x {keys} keys of its chunk", us, 2 * B * keys * G * D * e + 2 * B * H * D * e)
+    posd2 = i32([ctx - 1] * B)
+    us = _time_graph(lambda: ba.biased_attention(qd, kcd, vcd, V, seq_ids, posd2, qcud, table_d, cu_bd, 1 / math.sqrt(D), slopes, "causal",
+                                                 0, max_q_len=1), dev)
+    add(f"biased_attention, decode {B} x {ctx} keys (causal mask)", us, 2 * B * ctx * G * D * e + 2 * B * H * D * e)
+    # experts
+    logits, corr = f32(T, E + 1), f32(E) * 0.01
+    us = _time_graph(lambda: mm.route_softmax_topk(logits, E, top, 1.0, corr), dev)
+    add(f"route_softmax_topk ({E} experts, top {top})", us, T * (E + 1 + 2 * top) * 4)
+    wts, idx = mm.route_softmax_topk(logits, E, top, 1.0, corr)
+    us = _time_graph(lambda: mm.moe_plan(idx, E), dev)
+    add("moe_plan (one workgroup)", us, 3 * T * top * 4)
+    seg, row_of, src = mm.moe_plan(idx, E)
+    h, up, down = rnd(T, W), rnd(E, eff, W) / math.sqrt(W), rnd(E, W, eff) / math.sqrt(eff)
+    us = _time_graph(lambda: mm.grouped_linear(h, up, seg, T * top, src=src, act="relu2"), dev, launches=2)
+    add(f"grouped_linear up + squared ReLU ({T * top} rows, {W} -> {eff})", us, flops=2 * T * top * W * eff)
+    y1 = mm.grouped_linear(h, up, seg, T * top, src=src, act="relu2")
+    us = _time_graph(lambda: mm.grouped_linear(y1, down, seg, T * top), dev, launches=2)
+    add(f"grouped_linear down ({T * top} rows, {eff} -> {W})", us, flops=2 * T * top * W * eff)
+    y2, shared = mm.grouped_linear(y1, down, seg, T * top), rnd(T, W)
+    us = _time_graph(lambda: mm.moe_combine(y2, row_of, wts, shared, logits[:, E:]), dev)
+    add("moe_combine (+ gated shared expert)", us, T * W * (top + 2) * e)
+    # decode-sized expert products: B tokens, weights of the chosen experts stream once
+    hd = rnd(B, W)
+    wd, idd = mm.route_softmax_topk(logits[:B].contiguous(), E, top, 1.0, corr)
+    segd, rowd, srcd = mm.moe_plan(idd, E)
+    us = _time_graph(lambda: mm.grouped_linear(hd, up, segd, B * top, src=srcd, act="relu2"), dev)
+    used = int(torch.unique(idd).numel())
+    add(f"grouped_linear up, decode ({B} tokens, {used} experts' weights)", us, used * eff * W * e)
+    rows["llama"] = _llama_rows(size_name, dtype, dev, T, n_seqs, B, ctx)
+    a = rnd(T * top, W)
+    bw = rnd(eff, W)
+    us = _time_graph(lambda: torch.matmul(a, bw.t()), dev, launches=2)
+    rows["llama"].append(_row(f"library GEMM of the expert products' size ({T * top} x {W} -> {eff})", us, flops=2 * T * top * W * eff))
+    rows["workload"] = {"prefill_tokens": T, "portions": n_seqs, "decode_batch": B, "decode_keys": ctx, "size": sz,
+                        "timing": "hipGraph of 10 (long kernels: 2) launches, mean of 3 replays, HIP events",
+                        "roofline": f"HBM {HBM_PEAK_GBS} GB/s, MFMA {MFMA_PEAK_TFLOPS} TFLOP/s dense bf16; algorithmic bytes / flops"}
+    return rows
+
+
+def run(dtype, dev, sizes=("w2048", "w4096"), design: str = "tetepel") -> dict:
     from hydrainfer_amd import _lib
     _lib.lib(); _lib.mix_lib()
     res = {"throughput": {}, "kernels": {}}
+    table = {"tetepel": kernel_table, "kezolix": kezolix_kernel_table}[design]
     for s in sizes:
-        res["throughput"][s] = throughput(s, dtype, dev)
-        res["kernels"][s] = kernel_table(s, dtype, dev)
+        res["throughput"][s] = throughput(s, dtype, dev, design=design)
+        res["kernels"][s] = table(s, dtype, dev)
     return res

@@ -376,10 +376,49 @@ def test_attention_kernel_edges_far_keys_and_page_borders(H, G, D, V, mask, size
         pos = torch.tensor(sum(q_pos, []), dtype=torch.int32, device=DEV)
         tok_seq = torch.tensor(sum([[s] * len(p) for s, p in enumerate(q_pos)], []), dtype=torch.int32, device=DEV)
         q_cu = torch.tensor([0, 40, 73, 74], dtype=torch.int32, device=DEV)
-        out = biased_attention(q, kc, vc, V, tok_seq, pos, q_cu, table, cu, scale, _dev(slopes), mask, size, max_q_len=40, kv_heads=G)
-        _close(out, torch.cat(ref), tol, f"attention {mask} {dtype}")
+        for form, max_kv in (("auto", 0), ("auto", 150), ("rows", 0)):      # (with the keys' count known the tile form may split them)
+            out = biased_attention(q, kc, vc, V, tok_seq, pos, q_cu, table, cu, scale, _dev(slopes), mask, size, max_q_len=40,
+                                   kv_heads=G, max_kv_len=max_kv, form=form)
+            _close(out, torch.cat(ref), tol, f"attention {mask} {dtype} {form} {max_kv}")
         out = biased_attention(q, kc, vc, V, tok_seq, pos, q_cu, table, cu, scale, None, mask, size, max_q_len=40)
         assert (out.float().cpu() - torch.cat(ref).float()).abs().max() > 1e-3, "the distance bias changes the result"
+
+
+@pytest.mark.parametrize("mask,size", [("causal", 0), ("chunk", 300), ("window", 257)])
+def test_attention_tile_form_splits_the_keys_of_decode_steps(mask, size):
+    """Single decoded tokens of sequences of unequal length: few row tiles, so every tile's keys are dealt to several waves
+    and merged; one far key stands out."""
+    from hydrainfer_amd._C.kernel.biased_attn import biased_attention
+    g = torch.Generator().manual_seed(size)
+    H, G, D, V, bs, scale = 8, 2, 64, 96, 16, 0.2
+    lens = [700, 33, 1, 512, 301]
+    slopes = oracle.head_slopes(H)
+    ks = [torch.randn(n, G, D, generator=g).to(torch.bfloat16) for n in lens]
+    vs = [torch.randn(n, G, V, generator=g).to(torch.bfloat16) for n in lens]
+    qs = torch.randn(len(lens), H, D, generator=g).to(torch.bfloat16)
+    ks[0][5] *= 4.0
+    kc, vc, table, cu = _paged(ks, vs, bs, G, max(D, V), 6, torch.bfloat16)
+    ref = []
+    for s, n in enumerate(lens):
+        i, jj = n - 1, torch.arange(n)
+        see = jj <= i
+        if mask == "chunk":
+            see &= (jj // size) == (i // size)
+        if mask == "window":
+            see &= i - jj < size
+        out = torch.zeros(H, V, dtype=torch.float64)
+        for h in range(H):
+            gk = h // (H // G)
+            sc = ks[s][:, gk].double() @ qs[s, h].double() * scale - slopes[h] * (i - jj).double()
+            out[h] = torch.softmax(sc.masked_fill(~see, float("-inf")), dim=-1) @ vs[s][:, gk].double()
+        ref.append(out)
+    n = len(lens)
+    pos = torch.tensor([x - 1 for x in lens], dtype=torch.int32, device=DEV)
+    ids = torch.arange(n, dtype=torch.int32, device=DEV)
+    q_cu = torch.arange(n + 1, dtype=torch.int32, device=DEV)
+    out = biased_attention(_dev(qs, torch.bfloat16), kc, vc, V, ids, pos, q_cu, table, cu, scale, _dev(slopes), mask, size,
+                           max_q_len=1, max_kv_len=max(lens))
+    _close(out, torch.stack(ref), 3e-2, f"decode with key splits, {mask}")
 
 
 def test_query_key_norm_over_all_heads_and_cache_rows():
