@@ -37,9 +37,11 @@ def gated_recurrence(q_pre: Tensor, f_pre: Tensor, v: Tensor, f_bias: Tensor, lo
             raise _lib.HydraHipError(f"gated_recurrence: {name} must be contiguous int32 [{n}]")
     out = torch.empty((T, heads * vdim), dtype=dt, device=q_pre.device)
     base = st.data_ptr() + 4 * state_row * st.stride(1)
+    n_ws = _lib.mix_lib().hxm_gated_recurrence_workspace(T, int(heads), int(dim), int(vdim))
+    ws = torch.empty(max(n_ws, 1), dtype=torch.float32, device=q_pre.device)      # partial results of the key channels' parts
     _lib.mix_check(_lib.mix_lib().hxm_gated_recurrence(
         out.data_ptr(), q_pre.data_ptr(), q_pre.stride(0), f_pre.data_ptr(), f_pre.stride(0), v.data_ptr(), v.stride(0),
         f_bias.data_ptr(), low.data_ptr(), norm_w.data_ptr(), float(eps), base, st.stride(0), q_cu.data_ptr(),
-        positions.data_ptr(), seq.slots.data_ptr(), n_seq, int(heads), int(dim), int(vdim), _lib._DTYPE[dt],
-        _lib.current_stream()), "gated_recurrence")
+        positions.data_ptr(), seq.slots.data_ptr(), n_seq, T, int(heads), int(dim), int(vdim), ws.data_ptr(), n_ws,
+        _lib._DTYPE[dt], _lib.current_stream()), "gated_recurrence")
     return out

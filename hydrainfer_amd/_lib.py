@@ -278,9 +278,10 @@ _MIX_SIGNATURES = {
                                    c_int32, c_int, c_void_p]),
     "hxm_moe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64,
                                 c_int, c_void_p]),
+    "hxm_gated_recurrence_workspace": (c_int64, [c_int64, c_int32, c_int32, c_int32]),
     "hxm_gated_recurrence": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
-                                     c_float, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32,
-                                     c_int, c_void_p]),
+                                     c_float, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32,
+                                     c_int32, c_void_p, c_int64, c_int, c_void_p]),
     "hxm_qk_norm_cache": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                   c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int,
                                   c_void_p]),

@@ -5,6 +5,7 @@
 // (all heads at once), keys and values straight into the cache.
 #include <cfloat>
 #include "attn_common.h"
+#include "mix_rows.h"
 #include "../../include/hydra_mix.h"
 
 namespace hxm {
@@ -16,15 +17,8 @@ namespace {
 
 using namespace hx;
 
-__device__ __forceinline__ float block_sum4(float v, float* part) {
-  v = wave_sum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = v;
-  __syncthreads();
-  return part[0] + part[1] + part[2] + part[3];
-}
-
-// one workgroup per token
+// one workgroup per token.  vec: every offset, size, stride and pointer lets a lane move four elements at a time (and a
+// head's key / value rows are multiples of four)
 template <typename A>
 __global__ __launch_bounds__(256) void qk_norm_cache_kernel(const typename A::storage* __restrict__ proj, int64_t proj_stride,
                                                             int64_t q_off, int64_t q_size, int64_t k_off, int64_t k_size,
@@ -34,44 +28,73 @@ __global__ __launch_bounds__(256) void qk_norm_cache_kernel(const typename A::st
                                                             const int32_t* __restrict__ slot_ids,
                                                             typename A::storage* __restrict__ key_cache,
                                                             typename A::storage* __restrict__ value_cache,
-                                                            int64_t cache_row_stride, int64_t head_stride, int kv_heads) {
-  __shared__ float part[4];
+                                                            int64_t cache_row_stride, int64_t head_stride, int kv_heads, int vec) {
+  __shared__ float part[8];
   const int64_t t = blockIdx.x;
   const typename A::storage* row = proj + t * proj_stride;
-  {
-    float inv = 1.f;
-    if (q_w) {
-      float ss = 0.f;
-      for (int64_t i = threadIdx.x; i < q_size; i += 256) {
+  const int step = vec ? 4 : 1;
+  float ss[2] = {0.f, 0.f};      // sums of squares of the query and of the key projection, one pass
+  if (q_w) {
+    for (int64_t i = (int64_t)threadIdx.x * step; i < q_size; i += 256 * step) {
+      if (vec) {
+        const f32x4 v = Row4<A>::load(row + q_off + i);
+        ss[0] += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+      } else {
         const float v = A::to_float(row[q_off + i]);
-        ss += v * v;
+        ss[0] += v * v;
       }
-      inv = 1.0f / sqrtf(block_sum4(ss, part) / (float)q_size + eps);
     }
-    for (int64_t i = threadIdx.x; i < q_size; i += 256) {
-      const float v = A::to_float(row[q_off + i]);
-      q_out[t * q_size + i] = q_w ? A::from_float(v * inv * q_w[i]) : row[q_off + i];
+  }
+  if (k_w) {
+    for (int64_t i = (int64_t)threadIdx.x * step; i < k_size; i += 256 * step) {
+      if (vec) {
+        const f32x4 v = Row4<A>::load(row + k_off + i);
+        ss[1] += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+      } else {
+        const float v = A::to_float(row[k_off + i]);
+        ss[1] += v * v;
+      }
+    }
+  }
+  if (q_w || k_w) block_sums<2>(ss, part);
+  const float q_inv = 1.0f / sqrtf(ss[0] / (float)q_size + eps);
+  for (int64_t i = (int64_t)threadIdx.x * step; i < q_size; i += 256 * step) {
+    if (vec) {
+      f32x4 v = Row4<A>::load(row + q_off + i);
+      if (q_w) {
+        const f32x4 w = *reinterpret_cast<const f32x4*>(q_w + i);
+        v = f32x4{v[0] * q_inv * w[0], v[1] * q_inv * w[1], v[2] * q_inv * w[2], v[3] * q_inv * w[3]};
+      }
+      Row4<A>::store(q_out + t * q_size + i, v);
+    } else {
+      q_out[t * q_size + i] = q_w ? A::from_float(A::to_float(row[q_off + i]) * q_inv * q_w[i]) : row[q_off + i];
     }
   }
   if (k_size <= 0) return;
   const int64_t slot = slot_ids[t];
-  float inv = 1.f;
-  if (k_w) {
-    float ss = 0.f;
-    for (int64_t i = threadIdx.x; i < k_size; i += 256) {
-      const float v = A::to_float(row[k_off + i]);
-      ss += v * v;
-    }
-    inv = 1.0f / sqrtf(block_sum4(ss, part) / (float)k_size + eps);
-  }
   if (slot < 0) return;
+  const float k_inv = 1.0f / sqrtf(ss[1] / (float)k_size + eps);
   const int64_t kd = k_size / kv_heads, vd = v_size / kv_heads;
-  for (int64_t i = threadIdx.x; i < k_size; i += 256) {
-    const float v = A::to_float(row[k_off + i]);
-    key_cache[slot * cache_row_stride + (i / kd) * head_stride + i % kd] = k_w ? A::from_float(v * inv * k_w[i]) : row[k_off + i];
+  typename A::storage* kr = key_cache + slot * cache_row_stride;
+  typename A::storage* vr = value_cache + slot * cache_row_stride;
+  for (int64_t i = (int64_t)threadIdx.x * step; i < k_size; i += 256 * step) {
+    const int64_t at = (i / kd) * head_stride + i % kd;
+    if (vec) {
+      f32x4 v = Row4<A>::load(row + k_off + i);
+      if (k_w) {
+        const f32x4 w = *reinterpret_cast<const f32x4*>(k_w + i);
+        v = f32x4{v[0] * k_inv * w[0], v[1] * k_inv * w[1], v[2] * k_inv * w[2], v[3] * k_inv * w[3]};
+      }
+      Row4<A>::store(kr + at, v);
+    } else {
+      kr[at] = k_w ? A::from_float(A::to_float(row[k_off + i]) * k_inv * k_w[i]) : row[k_off + i];
+    }
   }
-  for (int64_t i = threadIdx.x; i < v_size; i += 256)
-    value_cache[slot * cache_row_stride + (i / vd) * head_stride + i % vd] = row[v_off + i];
+  for (int64_t i = (int64_t)threadIdx.x * step; i < v_size; i += 256 * step) {
+    const int64_t at = (i / vd) * head_stride + i % vd;
+    if (vec) Row4<A>::store(vr + at, Row4<A>::load(row + v_off + i));
+    else vr[at] = row[v_off + i];
+  }
 }
 
 // the wave's LDS writes so far are visible to all its lanes
@@ -253,9 +276,8 @@ __global__ __launch_bounds__(256) void biased_attn_tile_kernel(hxm_biased_attn_a
   }
   const int bs = a.block_size;
   const int bshift = (bs & (bs - 1)) == 0 ? __ffs(bs) - 1 : -1;
-  for (int key0 = k_begin; key0 <= k_end; key0 += 32) {
-    // half a chunk's rows, this lane's part: key 16 s + c, columns 32 kk + 8 g .. + 7
-    u16x8 kf[2][KK], vf[2][KK];
+  // a chunk's key or value rows, this lane's part: key 16 s + c, columns 32 kk + 8 g .. + 7
+  auto fetch = [&](int key0, const u16* base, int width, u16x8 (&f)[2][KK]) __attribute__((always_inline)) {
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       const int key = min(key0 + 16 * s + c, k_max);        // (a key past the last one repeats it; masked below)
@@ -264,20 +286,24 @@ __global__ __launch_bounds__(256) void biased_attn_tile_kernel(hxm_biased_attn_a
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
         const int col = 32 * kk + 8 * g;
-        kf[s][kk] = col < D ? *reinterpret_cast<const u16x8*>(kc + off + col) : zero8;
-        vf[s][kk] = col < V ? *reinterpret_cast<const u16x8*>(vc + off + col) : zero8;
+        f[s][kk] = col < width ? *reinterpret_cast<const u16x8*>(base + off + col) : zero8;
       }
     }
+  };
+  // One register set each for keys and values: a chunk's values are asked for before its scores are multiplied, and the
+  // next chunk's keys as soon as the scores are done — both loads are in flight behind the softmax and the products.
+  u16x8 kf[2][KK], vf[2][KK];
+  if (k_begin <= k_end) fetch(k_begin, kc, D, kf);
+  for (int key0 = k_begin; key0 <= k_end; key0 += 32) {
+    fetch(key0, vc, V, vf);
     f32x4 sc[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       sc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kk = 0; kk < KK; ++kk) {
-        sc[s] = Mfma<BF16>::mma(qf[kk], kf[s][kk], sc[s]);
-        *reinterpret_cast<u16x8*>(img + (16 * s + c) * RS + (32 * kk + 8 * g) * 2) = vf[s][kk];
-      }
+      for (int kk = 0; kk < KK; ++kk) sc[s] = Mfma<BF16>::mma(qf[kk], kf[s][kk], sc[s]);
     }
+    if (key0 + 32 <= k_end) fetch(key0 + 32, kc, D, kf);
     // softmax of the rows 4 g + i over this chunk (sc[s][i] is key key0 + 16 s + c)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -311,6 +337,10 @@ __global__ __launch_bounds__(256) void biased_attn_tile_kernel(hxm_biased_attn_a
       pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3)] = BF16::from_float(p[0]);
       pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3) + 4] = BF16::from_float(p[1]);
     }
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int kk = 0; kk < KK; ++kk) *reinterpret_cast<u16x8*>(img + (16 * s + c) * RS + (32 * kk + 8 * g) * 2) = vf[s][kk];
     wave_lds_sync();
     // O += P V: A = P[row c][slots 8 g ..], B = the image's column 16 n + c at the keys of those slots
     u16x8 pf;
@@ -434,16 +464,23 @@ extern "C" int hxm_qk_norm_cache(const void* proj, int64_t proj_stride, int64_t 
   }
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)n_tokens), block(256);
+  const uintptr_t es = dtype == HX_F32 ? 4 : 2;
+  auto by4 = [&](const void* p) { return ((uintptr_t)p % (4 * es)) == 0; };
+  int vec = q_off % 4 == 0 && q_size % 4 == 0 && proj_stride % 4 == 0 && by4(proj) && by4(q_out) &&
+            (!q_w || (uintptr_t)q_w % 16 == 0);
+  if (k_size > 0)
+    vec = vec && k_off % 4 == 0 && v_off % 4 == 0 && (k_size / kv_heads) % 4 == 0 && (v_size / kv_heads) % 4 == 0 &&
+          cache_row_stride % 4 == 0 && head_stride % 4 == 0 && by4(key_cache) && by4(value_cache) && (!k_w || (uintptr_t)k_w % 16 == 0);
   switch (dtype) {
     case HX_F32:
       qk_norm_cache_kernel<F32><<<grid, block, 0, s>>>((const float*)proj, proj_stride, q_off, q_size, k_off, k_size, v_off, v_size,
                                                        q_w, k_w, eps, (float*)q_out, slot_ids, (float*)key_cache, (float*)value_cache,
-                                                       cache_row_stride, head_stride, kv_heads);
+                                                       cache_row_stride, head_stride, kv_heads, vec);
       break;
     case HX_BF16:
       qk_norm_cache_kernel<BF16><<<grid, block, 0, s>>>((const u16*)proj, proj_stride, q_off, q_size, k_off, k_size, v_off, v_size,
                                                         q_w, k_w, eps, (u16*)q_out, slot_ids, (u16*)key_cache, (u16*)value_cache,
-                                                        cache_row_stride, head_stride, kv_heads);
+                                                        cache_row_stride, head_stride, kv_heads, vec);
       break;
     default: return HX_ERR_DTYPE;
   }

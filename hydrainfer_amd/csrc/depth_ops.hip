@@ -3,7 +3,7 @@
 // joins the stack of levels, the depth-weighted average of the levels becomes the next input, the next sublayer's input
 // is normed), and the PolyNorm / squared-ReLU activations.  One 256-thread workgroup per row, the row staged in LDS,
 // all arithmetic in float; only what a matrix product reads or writes has the activation dtype.
-#include "hx_common.h"
+#include "mix_rows.h"
 #include "../../include/hydra_mix.h"
 
 namespace hxm {
@@ -109,31 +109,55 @@ __global__ __launch_bounds__(256) void depth_norm_kernel(hxm_depth_norm_args a) 
   }
 }
 
+// vec: rows let a lane move four elements at a time (n, strides and pointers multiples of four elements)
 template <typename A>
 __global__ __launch_bounds__(256) void poly_norm_kernel(typename A::storage* __restrict__ out, int64_t out_stride,
                                                         const typename A::storage* __restrict__ z, int64_t z_stride,
-                                                        const float* __restrict__ coef, float eps, int64_t n) {
+                                                        const float* __restrict__ coef, float eps, int64_t n, int vec) {
   extern __shared__ float lds[];
   float* buf = lds;
-  float* part = lds + n;
+  float* part = lds + n;       // [12]
   const int64_t row = blockIdx.x;
-  float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-  for (int64_t i = threadIdx.x; i < n; i += 256) {
-    const float v = A::to_float(z[row * z_stride + i]);
-    buf[i] = v;
-    const float v2 = v * v;
-    s2 += v2;
-    s4 += v2 * v2;
-    s6 += v2 * v2 * v2;
+  float s[3] = {0.f, 0.f, 0.f};
+  if (vec) {
+    for (int64_t i = (int64_t)threadIdx.x * 4; i < n; i += 1024) {
+      const f32x4 v = Row4<A>::load(z + row * z_stride + i);
+      *reinterpret_cast<f32x4*>(buf + i) = v;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const float v2 = v[k] * v[k];
+        s[0] += v2;
+        s[1] += v2 * v2;
+        s[2] += v2 * v2 * v2;
+      }
+    }
+  } else {
+    for (int64_t i = threadIdx.x; i < n; i += 256) {
+      const float v = A::to_float(z[row * z_stride + i]);
+      buf[i] = v;
+      const float v2 = v * v;
+      s[0] += v2;
+      s[1] += v2 * v2;
+      s[2] += v2 * v2 * v2;
+    }
   }
-  s2 = block_sum(s2, part);
-  s4 = block_sum(s4, part);
-  s6 = block_sum(s6, part);
-  const float r1 = coef[0] / sqrtf(s2 / (float)n + eps), r2 = coef[1] / sqrtf(s4 / (float)n + eps),
-              r3 = coef[2] / sqrtf(s6 / (float)n + eps), c3 = coef[3];
-  for (int64_t i = threadIdx.x; i < n; i += 256) {
-    const float v = buf[i];
-    out[row * out_stride + i] = A::from_float(v * r1 + v * v * r2 + v * v * v * r3 + c3);
+  block_sums<3>(s, part);
+  const float r1 = coef[0] / sqrtf(s[0] / (float)n + eps), r2 = coef[1] / sqrtf(s[1] / (float)n + eps),
+              r3 = coef[2] / sqrtf(s[2] / (float)n + eps), c3 = coef[3];
+  // (a thread reads back the elements of buf it wrote itself)
+  if (vec) {
+    for (int64_t i = (int64_t)threadIdx.x * 4; i < n; i += 1024) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(buf + i);
+      f32x4 o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] = v[k] * r1 + v[k] * v[k] * r2 + v[k] * v[k] * v[k] * r3 + c3;
+      Row4<A>::store(out + row * out_stride + i, o);
+    }
+  } else {
+    for (int64_t i = threadIdx.x; i < n; i += 256) {
+      const float v = buf[i];
+      out[row * out_stride + i] = A::from_float(v * r1 + v * v * r2 + v * v * v * r3 + c3);
+    }
   }
 }
 
@@ -198,13 +222,15 @@ extern "C" int hxm_poly_norm(void* out, int64_t out_stride, const void* z, int64
   if (rows == 0) return HX_OK;
   if (!out || !z || !coef) return HX_ERR_NULL;
   if (out_stride < n || z_stride < n) return HX_ERR_STRIDE;
-  const size_t lds = ((size_t)n + 4) * sizeof(float);
+  const size_t lds = ((size_t)n + 12) * sizeof(float);
   if (lds > 64 * 1024) return HX_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)rows), block(256);
+  const int es = dtype == HX_F32 ? 4 : 2;
+  const int vec = n % 4 == 0 && out_stride % 4 == 0 && z_stride % 4 == 0 && ((uintptr_t)out % (4 * es)) == 0 && ((uintptr_t)z % (4 * es)) == 0;
   switch (dtype) {
-    case HX_F32: poly_norm_kernel<F32><<<grid, block, lds, s>>>((float*)out, out_stride, (const float*)z, z_stride, coef, eps, n); break;
-    case HX_BF16: poly_norm_kernel<BF16><<<grid, block, lds, s>>>((u16*)out, out_stride, (const u16*)z, z_stride, coef, eps, n); break;
+    case HX_F32: poly_norm_kernel<F32><<<grid, block, lds, s>>>((float*)out, out_stride, (const float*)z, z_stride, coef, eps, n, vec); break;
+    case HX_BF16: poly_norm_kernel<BF16><<<grid, block, lds, s>>>((u16*)out, out_stride, (const u16*)z, z_stride, coef, eps, n, vec); break;
     default: return HX_ERR_DTYPE;
   }
   return hxm::check_launch();

@@ -2,10 +2,13 @@
 // decides what is written:  f = low + (1 - low) sigmoid(f_pre + b),  S <- diag(f) S + (1 - f) v^T,  o = S^T silu(q_pre),
 // then o is RMS-normed over the head's value channels.  Gates, state and sums are float.
 //
-// One workgroup per (sequence, head).  A lane owns one value channel (column of S); the key channels (rows of S) are
-// dealt to `n_dg` groups of waves, DR rows each, held in registers.  Rows of S evolve independently, so the groups never
-// talk during the scan: they leave partial o's in LDS, a chunk of tokens at a time, which are then summed and normed.
-// The gates of a chunk are worked out once, by all threads, into LDS.  Two barriers per chunk of tokens.
+// The scan: a workgroup takes (sequence, head, 64 value channels, a part of the key channels).  A lane owns one value
+// channel (column of S); the part's key channels (rows of S) are dealt to the workgroup's waves, DR rows each, held in
+// registers.  Rows of S evolve independently, so nothing is exchanged during the scan: per chunk of 16 tokens the gates of
+// the part's rows are worked out once into LDS (f and silu(q) side by side, read back 16 bytes at a time), a lane's values
+// of the chunk are loaded into registers before the scan starts (the serial chain holds no global load), the waves'
+// partial o's are summed through LDS and leave for a float workspace [parts][tokens][heads * vdim].  A second kernel — one
+// wave per (token, head) — sums the parts and norms over the head's value channels.
 #include "hx_common.h"
 #include "../../include/hydra_mix.h"
 
@@ -17,6 +20,9 @@ int check_launch();
 namespace {
 
 using namespace hx;
+
+constexpr int kTC = 16;          // tokens a chunk
+constexpr int kMaxWaves = 8;     // waves a workgroup
 
 struct RecArgs {
   void* out;
@@ -32,26 +38,26 @@ struct RecArgs {
   const int32_t* q_cu;
   const int32_t* positions;
   const int32_t* slots;
-  int32_t heads, dim, vdim, n_cw, n_dg, chunk;
+  float* ws;                     // [n_parts][n_tokens][heads * vdim]
+  int64_t n_tokens;
+  int32_t heads, dim, vdim, n_cw, n_parts, n_waves;
   float eps;
 };
 
 template <typename A, int DR>
-__global__ __launch_bounds__(1024) void gated_recurrence_kernel(RecArgs a) {
-  extern __shared__ float lds[];
+__global__ __launch_bounds__(64 * kMaxWaves) void gated_recurrence_scan_kernel(RecArgs a) {
+  __shared__ __attribute__((aligned(16))) float gates[kTC * kMaxWaves * DR * 2];      // [token][row of the part][f, silu(q)]
+  __shared__ float po[kTC * kMaxWaves * 64];                                           // [token][wave][lane]
   typedef typename A::storage T;
   const int seq = blockIdx.x, head = blockIdx.y;
-  const int D = a.dim, V = a.vdim, TC = a.chunk;
-  const int n_waves = a.n_cw * a.n_dg, n_threads = n_waves * 64;
+  const int cw = blockIdx.z % a.n_cw, part = blockIdx.z / a.n_cw;
+  const int D = a.dim, V = a.vdim, NW = a.n_waves;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int cw = wave % a.n_cw, dg = wave / a.n_cw;
   const int col = cw * 64 + lane;
   const bool col_ok = col < V;
-  const int d0 = dg * DR;
-  const int Vp = a.n_cw * 64;
-  float* gq = lds;                         // [TC][D]   silu(q_pre)
-  float* gf = gq + TC * D;                 // [TC][D]   f
-  float* po = gf + TC * D;                 // [TC][n_dg][Vp]   partial o's
+  const int rows_part = NW * DR;                 // key channels of this part (the last part may reach past D: f = 1, q = 0)
+  const int part_d0 = part * rows_part;
+  const int d0 = part_d0 + wave * DR;
   const int t_begin = a.q_cu[seq], t_end = a.q_cu[seq + 1];
   if (t_end <= t_begin) return;
   float* slot = a.state + (int64_t)a.slots[seq] * a.slot_stride + (int64_t)head * D * V;
@@ -65,51 +71,78 @@ __global__ __launch_bounds__(1024) void gated_recurrence_kernel(RecArgs a) {
   const T* qp = (const T*)a.q_pre + head * D;
   const T* fp = (const T*)a.f_pre + head * D;
   const T* vp = (const T*)a.v + head * V;
-  T* op = (T*)a.out + head * V;
   const float* fb = a.f_bias + head * D;
   const float* lw = a.low + head * D;
-  for (int t0 = t_begin; t0 < t_end; t0 += TC) {
-    const int nt = t_end - t0 < TC ? t_end - t0 : TC;
-    for (int i = threadIdx.x; i < nt * D; i += n_threads) {
-      const int tt = i / D, d = i - tt * D;
-      const float qv = A::to_float(qp[(int64_t)(t0 + tt) * a.q_stride + d]);
-      const float fv = A::to_float(fp[(int64_t)(t0 + tt) * a.f_stride + d]) + fb[d];
-      const float l = lw[d];
-      gq[tt * D + d] = qv / (1.0f + expf(-qv));
-      gf[tt * D + d] = l + (1.0f - l) / (1.0f + expf(-fv));
-    }
-    __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
-      const float vv = col_ok ? A::to_float(vp[(int64_t)(t0 + tt) * a.v_stride + col]) : 0.f;
-      const float* q_t = gq + tt * D + d0;
-      const float* f_t = gf + tt * D + d0;
-      float o = 0.f;
+  float* wo = a.ws + (int64_t)part * a.n_tokens * (a.heads * V) + head * V;
+  const int n_threads = NW * 64;
+  // the pre-activations a thread turns into gates (element e of a chunk: token e / rows_part, row e % rows_part) and the
+  // lane's values, asked for one chunk ahead
+  constexpr int EPT = kTC * DR / 64;
+  float qn[EPT], fn[EPT], vn[kTC];
+  auto fetch = [&](int t0) __attribute__((always_inline)) {
+    const int nt = t_end - t0 < kTC ? t_end - t0 : kTC;
 #pragma unroll
-      for (int r = 0; r < DR; ++r) {
-        if (d0 + r < D) {
-          const float f = f_t[r];
-          S[r] = f * S[r] + (1.0f - f) * vv;
-          o += q_t[r] * S[r];
-        }
+    for (int e = 0; e < EPT; ++e) {
+      const int i = threadIdx.x + e * n_threads;
+      const int tt = i / rows_part, d = part_d0 + i - tt * rows_part;
+      const bool ok = tt < nt && d < D;
+      qn[e] = ok ? A::to_float(qp[(int64_t)(t0 + tt) * a.q_stride + d]) : 0.f;
+      fn[e] = ok ? A::to_float(fp[(int64_t)(t0 + tt) * a.f_stride + d]) : 0.f;
+    }
+#pragma unroll
+    for (int tt = 0; tt < kTC; ++tt)
+      vn[tt] = (col_ok && tt < nt) ? A::to_float(vp[(int64_t)(t0 + tt) * a.v_stride + col]) : 0.f;
+  };
+  fetch(t_begin);
+  for (int t0 = t_begin; t0 < t_end; t0 += kTC) {
+    const int nt = t_end - t0 < kTC ? t_end - t0 : kTC;
+    float vv[kTC];
+#pragma unroll
+    for (int tt = 0; tt < kTC; ++tt) vv[tt] = vn[tt];
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int i = threadIdx.x + e * n_threads;
+      const int tt = i / rows_part, d = part_d0 + i - tt * rows_part;
+      float q = 0.f, f = 1.f;
+      if (tt < nt && d < D) {
+        const float qv = qn[e], fv = fn[e] + fb[d], l = lw[d];
+        q = qv / (1.0f + expf(-qv));
+        f = l + (1.0f - l) / (1.0f + expf(-fv));
       }
-      po[(tt * a.n_dg + dg) * Vp + col] = o;
+      gates[2 * i] = f;
+      gates[2 * i + 1] = q;
+    }
+    if (t0 + kTC < t_end) fetch(t0 + kTC);
+    __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < kTC; ++tt) {
+      if (tt < nt) {
+        const f32x4* g4 = reinterpret_cast<const f32x4*>(gates + 2 * (tt * rows_part + wave * DR));
+        const float v = vv[tt];
+        float o = 0.f;
+#pragma unroll
+        for (int r2 = 0; r2 < DR / 2; ++r2) {
+          const f32x4 g = g4[r2];                   // f, silu(q) of two rows
+          S[2 * r2] = v + g[0] * (S[2 * r2] - v);   // = f S + (1 - f) v
+          o += g[1] * S[2 * r2];
+          S[2 * r2 + 1] = v + g[2] * (S[2 * r2 + 1] - v);
+          o += g[3] * S[2 * r2 + 1];
+        }
+        po[(tt * kMaxWaves + wave) * 64 + lane] = o;
+      }
     }
     __syncthreads();
-    // sum the groups' partial o's, norm over the head's value channels: a wave takes a token at a time
-    for (int tt = wave; tt < nt; tt += n_waves) {
-      float ss = 0.f;
-      for (int c = lane; c < V; c += 64) {
+    // the waves' partial o's of the chunk, summed: thread (tt, lane) pairs dealt over the workgroup
+    for (int i = threadIdx.x; i < nt * 64; i += n_threads) {
+      const int tt = i >> 6, ln = i & 63, c = cw * 64 + ln;
+      if (c < V) {
         float o = 0.f;
-        for (int g = 0; g < a.n_dg; ++g) o += po[(tt * a.n_dg + g) * Vp + c];
-        po[(tt * a.n_dg) * Vp + c] = o;      // (this lane alone reads and writes column c of token tt)
-        ss += o * o;
+        for (int w = 0; w < NW; ++w) o += po[(tt * kMaxWaves + w) * 64 + ln];
+        wo[(int64_t)(t0 + tt) * (a.heads * V) + c] = o;
       }
-      ss = wave_sum(ss);
-      const float inv = 1.0f / sqrtf(ss / (float)V + a.eps);
-      for (int c = lane; c < V; c += 64)
-        op[(int64_t)(t0 + tt) * (a.heads * V) + c] = A::from_float(po[(tt * a.n_dg) * Vp + c] * inv * a.norm_w[c]);
     }
-    // (the next chunk's gates go to gq / gf, which nobody reads any more; po is written again only after the next barrier)
+    // (the next chunk's gates are written while slow waves may still sum: they read po only; po is written again after
+    //  the next barrier)
   }
 #pragma unroll
   for (int r = 0; r < DR; ++r) {
@@ -118,67 +151,88 @@ __global__ __launch_bounds__(1024) void gated_recurrence_kernel(RecArgs a) {
   }
 }
 
+// one wave per (token, head): the parts summed, normed over the head's value channels, times norm_w
 template <typename A>
-int launch_recurrence(const RecArgs& a, int n_seq, int dr, size_t lds, hipStream_t s) {
-  const dim3 grid((unsigned)n_seq, (unsigned)a.heads), block((unsigned)(a.n_cw * a.n_dg * 64));
-#define HXM_REC(DR_)                                                                                                      \
-  do {                                                                                                                    \
-    if (lds > 48 * 1024) {                                                                                                \
-      hipError_t e = hipFuncSetAttribute((const void*)gated_recurrence_kernel<A, DR_>,                                    \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                           \
-      if (e != hipSuccess) {                                                                                              \
-        hxm::last_hip_error() = (int)e;                                                                                   \
-        return HX_ERR_HIP;                                                                                                \
-      }                                                                                                                   \
-    }                                                                                                                     \
-    gated_recurrence_kernel<A, DR_><<<grid, block, lds, s>>>(a);                                                          \
-  } while (0)
-  switch (dr) {
-    case 8: HXM_REC(8); break;
-    case 16: HXM_REC(16); break;
-    case 32: HXM_REC(32); break;
-    case 64: HXM_REC(64); break;
-    default: return HX_ERR_SHAPE;
+__global__ __launch_bounds__(256) void gated_recurrence_norm_kernel(RecArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (item >= a.n_tokens * a.heads) return;
+  const int V = a.vdim;
+  const int64_t HV = (int64_t)a.heads * V, at = (item / a.heads) * HV + (item % a.heads) * V;
+  float o[16];       // vdim <= 1024
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const int c = lane + 64 * k;
+    o[k] = 0.f;
+    if (c < V) {
+      for (int p = 0; p < a.n_parts; ++p) o[k] += a.ws[(int64_t)p * a.n_tokens * HV + at + c];
+      ss += o[k] * o[k];
+    }
   }
-#undef HXM_REC
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)V + a.eps);
+  typename A::storage* out = (typename A::storage*)a.out + at;
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const int c = lane + 64 * k;
+    if (c < V) out[c] = A::from_float(o[k] * inv * a.norm_w[c]);
+  }
+}
+
+// rows a wave holds, waves a workgroup, parts of the key channels
+void recurrence_layout(int dim, int& dr, int& n_waves, int& n_parts) {
+  dr = dim > 16 ? 8 : 4;      // (16 rows a wave: the unrolled scan of a chunk holds every gate it reads in registers — too many)
+  const int groups = (dim + dr - 1) / dr;
+  n_waves = groups < kMaxWaves ? groups : kMaxWaves;
+  n_parts = (groups + n_waves - 1) / n_waves;
+}
+
+template <typename A>
+int launch_recurrence(const RecArgs& a, int n_seq, int dr, hipStream_t s) {
+  const dim3 grid((unsigned)n_seq, (unsigned)a.heads, (unsigned)(a.n_cw * a.n_parts)), block((unsigned)(a.n_waves * 64));
+  switch (dr) {
+    case 4: gated_recurrence_scan_kernel<A, 4><<<grid, block, 0, s>>>(a); break;
+    default: gated_recurrence_scan_kernel<A, 8><<<grid, block, 0, s>>>(a); break;
+  }
+  gated_recurrence_norm_kernel<A><<<dim3((unsigned)((a.n_tokens * a.heads + 3) / 4)), dim3(256), 0, s>>>(a);
   return hxm::check_launch();
 }
 
 }  // namespace
 
+extern "C" int64_t hxm_gated_recurrence_workspace(int64_t n_tokens, int32_t heads, int32_t dim, int32_t vdim) {
+  if (n_tokens < 0 || heads < 1 || dim < 1 || vdim < 1) return 0;
+  int dr, n_waves, n_parts;
+  recurrence_layout(dim, dr, n_waves, n_parts);
+  return (int64_t)n_parts * n_tokens * heads * vdim;
+}
+
 extern "C" int hxm_gated_recurrence(void* out, const void* q_pre, int64_t q_stride, const void* f_pre, int64_t f_stride,
                                     const void* v, int64_t v_stride, const float* f_bias, const float* low,
                                     const float* norm_w, float eps, float* state, int64_t slot_stride, const int32_t* q_cu,
-                                    const int32_t* positions, const int32_t* slots, int32_t n_seq, int32_t heads, int32_t dim,
-                                    int32_t vdim, int dtype, void* stream) {
-  if (n_seq < 0 || heads < 1 || dim < 1 || vdim < 1 || dim > 1024 || vdim > 1024) return HX_ERR_SHAPE;
-  if (n_seq == 0) return HX_OK;
-  if (!out || !q_pre || !f_pre || !v || !f_bias || !low || !norm_w || !state || !q_cu || !positions || !slots) return HX_ERR_NULL;
+                                    const int32_t* positions, const int32_t* slots, int32_t n_seq, int64_t n_tokens,
+                                    int32_t heads, int32_t dim, int32_t vdim, float* ws, int64_t ws_floats, int dtype,
+                                    void* stream) {
+  if (n_seq < 0 || n_tokens < 0 || heads < 1 || dim < 1 || vdim < 1 || vdim > 1024 || heads > 65535) return HX_ERR_SHAPE;
+  if (n_seq == 0 || n_tokens == 0) return HX_OK;
+  if (!out || !q_pre || !f_pre || !v || !f_bias || !low || !norm_w || !state || !q_cu || !positions || !slots || !ws) return HX_ERR_NULL;
   if (slot_stride < (int64_t)heads * dim * vdim) return HX_ERR_STRIDE;
   RecArgs a;
   a.out = out; a.q_pre = q_pre; a.f_pre = f_pre; a.v = v;
   a.q_stride = q_stride; a.f_stride = f_stride; a.v_stride = v_stride;
   a.f_bias = f_bias; a.low = low; a.norm_w = norm_w; a.state = state; a.slot_stride = slot_stride;
-  a.q_cu = q_cu; a.positions = positions; a.slots = slots;
+  a.q_cu = q_cu; a.positions = positions; a.slots = slots; a.ws = ws; a.n_tokens = n_tokens;
   a.heads = heads; a.dim = dim; a.vdim = vdim; a.eps = eps;
-  a.n_cw = (vdim + 63) / 64;                       // waves across the value channels: 1 .. 16
-  // groups of key channels: as many as fit 16 waves, no fewer rows than 8 a group, no more than 64 (the registers)
-  int n_dg = 16 / a.n_cw;
-  while (n_dg > 1 && (dim + n_dg - 1) / n_dg < 8) --n_dg;
-  int rows = (dim + n_dg - 1) / n_dg;
-  if (rows > 64) return HX_ERR_SHAPE;              // dim * ceil(vdim / 64) <= 1024
-  const int dr = rows <= 8 ? 8 : rows <= 16 ? 16 : rows <= 32 ? 32 : 64;
-  n_dg = (dim + dr - 1) / dr;
-  a.n_dg = n_dg;
-  int chunk = 16;
-  auto lds_of = [&](int tc) { return (size_t)tc * (2 * (size_t)dim + (size_t)n_dg * a.n_cw * 64) * sizeof(float); };
-  while (chunk > 1 && lds_of(chunk) > 96 * 1024) chunk >>= 1;
-  if (lds_of(chunk) > 96 * 1024) return HX_ERR_SHAPE;
-  a.chunk = chunk;
+  a.n_cw = (vdim + 63) / 64;
+  int dr;
+  recurrence_layout(dim, dr, a.n_waves, a.n_parts);
+  if ((int64_t)a.n_cw * a.n_parts > 65535) return HX_ERR_SHAPE;
+  if (ws_floats < (int64_t)a.n_parts * n_tokens * heads * vdim) return HX_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
-    case HX_F32: return launch_recurrence<F32>(a, n_seq, dr, lds_of(chunk), s);
-    case HX_BF16: return launch_recurrence<BF16>(a, n_seq, dr, lds_of(chunk), s);
+    case HX_F32: return launch_recurrence<F32>(a, n_seq, dr, s);
+    case HX_BF16: return launch_recurrence<BF16>(a, n_seq, dr, s);
     default: return HX_ERR_DTYPE;
   }
 }

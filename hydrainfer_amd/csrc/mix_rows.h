@@ -1,0 +1,45 @@
+// mix_rows.h — helpers of the mix library's row kernels: four consecutive elements of an activation row as four floats,
+// and sums over a 256-thread workgroup.
+#pragma once
+#include "hx_common.h"
+
+namespace hx {
+
+template <typename A> struct Row4;
+template <> struct Row4<F32> {
+  static __device__ __forceinline__ f32x4 load(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+  static __device__ __forceinline__ void store(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+};
+template <> struct Row4<BF16> {
+  static __device__ __forceinline__ f32x4 load(const u16* p) {
+    const u16x4 b = *reinterpret_cast<const u16x4*>(p);
+    return f32x4{BF16::to_float(b[0]), BF16::to_float(b[1]), BF16::to_float(b[2]), BF16::to_float(b[3])};
+  }
+  static __device__ __forceinline__ void store(u16* p, f32x4 v) {
+    *reinterpret_cast<u16x4*>(p) = u16x4{BF16::from_float(v[0]), BF16::from_float(v[1]), BF16::from_float(v[2]), BF16::from_float(v[3])};
+  }
+};
+
+// true if p and the row stride (elements) let a lane move four elements of type T at a time
+template <typename T>
+inline bool rows_by_four(const void* p, int64_t stride) {
+  return (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T))) == 0 && stride % 4 == 0;
+}
+
+// sums of N values over the 256 threads of the workgroup; part: 4 * N floats of LDS.  Every thread ends with the sums; part
+// may be used again after the next barrier.
+template <int N>
+__device__ __forceinline__ void block_sums(float (&v)[N], float* part) {
+#pragma unroll
+  for (int n = 0; n < N; ++n) v[n] = wave_sum(v[n]);
+  __syncthreads();                       // the previous use of part is over
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) part[(threadIdx.x >> 6) * N + n] = v[n];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int n = 0; n < N; ++n) v[n] = part[n] + part[N + n] + part[2 * N + n] + part[3 * N + n];
+}
+
+}  // namespace hx

@@ -203,55 +203,94 @@ __global__ __launch_bounds__(256) void grouped_linear_kernel(typename A::storage
   }
 }
 
-// MFMA form (bfloat16, K a multiple of 32, rows 16-byte aligned): a workgroup of four waves takes 64 rows of one expert and
-// 64 output columns; wave w rows 16 w .. 16 w + 15, all 64 columns (four 16x16 accumulators).  Both operands of the
-// 16x16x32 MFMA are 16-byte pieces of K-contiguous rows, so they come straight from global memory: lane l holds
-// k 8 (l / 16) .. + 7 of row (A) or column (B) l % 16; the accumulator's lane l holds column l % 16 of rows 4 (l / 16) .. + 3.
-constexpr int kTM = 64, kTN = 64;
-__global__ __launch_bounds__(256) void grouped_linear_mfma_kernel(u16* __restrict__ y, const u16* __restrict__ x, int64_t x_stride,
-                                                                  const int32_t* __restrict__ src, const u16* __restrict__ w,
-                                                                  const int32_t* __restrict__ seg, int E, int64_t N, int64_t K,
-                                                                  int act) {
+// MFMA form (bfloat16, K a multiple of 8, rows 16-byte aligned): a workgroup of four waves takes TM rows of one expert and
+// TN output columns; the rows' inputs (gathered through src) and the expert's weight rows go through LDS in slices of 64
+// k — the next slice is on its way into registers while the current one is multiplied — and every wave multiplies its
+// (TM / WGM) x (TN / WGN) part with 16x16x32 MFMAs: lane l holds k 8 (l / 16) .. + 7 of row (A) or column (B) l % 16, the
+// accumulator's lane l column l % 16 of rows 4 (l / 16) .. + 3.  Rows of LDS are padded to 72 elements (144 bytes): the
+// sixteen rows a 16-byte read touches fall into different banks.
+constexpr int kKS = 64, kLDK = 72;
+template <int TM, int TN, int WGM, int WGN>
+__global__ __launch_bounds__(256) void grouped_linear_tiled_kernel(u16* __restrict__ y, const u16* __restrict__ x, int64_t x_stride,
+                                                                   const int32_t* __restrict__ src, const u16* __restrict__ w,
+                                                                   const int32_t* __restrict__ seg, int E, int64_t N, int64_t K,
+                                                                   int act) {
+  constexpr int FM = TM / WGM / 16, FN = TN / WGN / 16;
+  constexpr int PA = TM * 8 / 256, PB = TN * 8 / 256;      // 16-byte pieces of a slice a thread moves
+  __shared__ __attribute__((aligned(16))) u16 As[TM * kLDK];
+  __shared__ __attribute__((aligned(16))) u16 Bs[TN * kLDK];
   int e, row0, row1;
-  if (!find_tile(seg, E, kTM, blockIdx.y, e, row0, row1)) return;
+  if (!find_tile(seg, E, TM, blockIdx.y, e, row0, row1)) return;      // (the whole workgroup: no barrier is left waiting)
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int wrow0 = row0 + 16 * wave;
-  if (wrow0 >= row1) return;                                   // (no barriers in this kernel)
-  const int64_t col0 = (int64_t)blockIdx.x * kTN;
-  const int l16 = lane & 15, kq = lane >> 4;
-  const int arow = wrow0 + l16;
-  const bool a_ok = arow < row1;
-  const int64_t sr = a_ok ? (src ? (int64_t)src[arow] : (int64_t)arow) : 0;
-  const u16* ap = x + sr * x_stride + kq * 8;
+  const int wm0 = (wave / WGN) * (TM / WGM), wn0 = (wave % WGN) * (TN / WGN);
+  const int64_t col0 = (int64_t)blockIdx.x * TN;
   const u16* we = w + (int64_t)e * N * K;
-  const u16* bp[4];
-  bool b_ok[4];
-  for (int j = 0; j < 4; ++j) {
-    const int64_t c = col0 + 16 * j + l16;
-    b_ok[j] = c < N;
-    bp[j] = we + (b_ok[j] ? c : 0) * K + kq * 8;
-  }
-  f32x4 acc[4];
-  for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const bf16x8 zero = __builtin_bit_cast(bf16x8, u16x8{0, 0, 0, 0, 0, 0, 0, 0});
-  for (int64_t k0 = 0; k0 < K; k0 += 32) {
-    const bf16x8 av = a_ok ? __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8*>(ap + k0)) : zero;
+  const u16x8 zero8 = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  const u16* pa[PA];
+  const u16* pb[PB];
+  int ka[PA], kb[PB];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const bf16x8 bv = b_ok[j] ? __builtin_bit_cast(bf16x8, *reinterpret_cast<const u16x8*>(bp[j] + k0)) : zero;
-      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc[j], 0, 0, 0);
+  for (int p = 0; p < PA; ++p) {
+    const int idx = threadIdx.x + 256 * p, r = idx >> 3;
+    ka[p] = (idx & 7) * 8;
+    pa[p] = nullptr;
+    if (row0 + r < row1) pa[p] = x + (src ? (int64_t)src[row0 + r] : (int64_t)(row0 + r)) * x_stride + ka[p];
+  }
+#pragma unroll
+  for (int p = 0; p < PB; ++p) {
+    const int idx = threadIdx.x + 256 * p, c = idx >> 3;
+    kb[p] = (idx & 7) * 8;
+    pb[p] = col0 + c < N ? we + (col0 + c) * K + kb[p] : nullptr;
+  }
+  u16x8 ra[PA], rb[PB];
+  auto fetch = [&](int64_t k0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int p = 0; p < PA; ++p) ra[p] = (pa[p] && k0 + ka[p] < K) ? *reinterpret_cast<const u16x8*>(pa[p] + k0) : zero8;
+#pragma unroll
+    for (int p = 0; p < PB; ++p) rb[p] = (pb[p] && k0 + kb[p] < K) ? *reinterpret_cast<const u16x8*>(pb[p] + k0) : zero8;
+  };
+  f32x4 acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int l16 = lane & 15, kq = lane >> 4;
+  fetch(0);
+  for (int64_t k0 = 0; k0 < K; k0 += kKS) {
+#pragma unroll
+    for (int p = 0; p < PA; ++p) *reinterpret_cast<u16x8*>(As + ((threadIdx.x + 256 * p) >> 3) * kLDK + ka[p]) = ra[p];
+#pragma unroll
+    for (int p = 0; p < PB; ++p) *reinterpret_cast<u16x8*>(Bs + ((threadIdx.x + 256 * p) >> 3) * kLDK + kb[p]) = rb[p];
+    __syncthreads();
+    if (k0 + kKS < K) fetch(k0 + kKS);
+#pragma unroll
+    for (int ks = 0; ks < kKS / 32; ++ks) {
+      u16x8 af[FM], bf[FN];
+#pragma unroll
+      for (int i = 0; i < FM; ++i) af[i] = *reinterpret_cast<const u16x8*>(As + (wm0 + 16 * i + l16) * kLDK + 32 * ks + 8 * kq);
+#pragma unroll
+      for (int j = 0; j < FN; ++j) bf[j] = *reinterpret_cast<const u16x8*>(Bs + (wn0 + 16 * j + l16) * kLDK + 32 * ks + 8 * kq);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af[i]), __builtin_bit_cast(bf16x8, bf[j]),
+                                                              acc[i][j], 0, 0, 0);
     }
+    __syncthreads();
   }
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int64_t c = col0 + 16 * j + l16;
-    if (c >= N) continue;
+  for (int i = 0; i < FM; ++i)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int rr = wrow0 + 4 * kq + i;
-      if (rr < row1) y[(int64_t)rr * N + c] = BF16::from_float(act_apply(acc[j][i], act));
+    for (int j = 0; j < FN; ++j) {
+      const int64_t c = col0 + wn0 + 16 * j + l16;
+      if (c >= N) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int rr = row0 + wm0 + 16 * i + 4 * kq + r;
+        if (rr < row1) y[(int64_t)rr * N + c] = BF16::from_float(act_apply(acc[i][j][r], act));
+      }
     }
-  }
 }
 
 template <typename A>
@@ -310,11 +349,19 @@ extern "C" int hxm_grouped_linear(void* y, const void* x, int64_t x_stride, cons
   if (!y || !x || !w || !seg) return HX_ERR_NULL;
   if (x_stride < k_dim) return HX_ERR_STRIDE;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == HX_BF16 && k_dim % 32 == 0 && x_stride % 8 == 0 && aligned16(x) && aligned16(w)) {
-    const int64_t tiles = (max_rows + kTM - 1) / kTM + n_experts;      // every expert's rows start a tile of their own
+  if (dtype == HX_BF16 && k_dim % 8 == 0 && x_stride % 8 == 0 && aligned16(x) && aligned16(w)) {
+    // few rows an expert (decode steps): tiles of 32 rows, the four waves side by side over 128 columns; else 128 x 128
+    const bool small = max_rows <= (int64_t)32 * n_experts;
+    const int tm = small ? 32 : 128;
+    const int64_t tiles = (max_rows + tm - 1) / tm + n_experts;      // every expert's rows start a tile of their own
     if (tiles > 65535) return HX_ERR_SHAPE;
-    grouped_linear_mfma_kernel<<<dim3((unsigned)((n_dim + kTN - 1) / kTN), (unsigned)tiles), dim3(256), 0, s>>>(
-        (u16*)y, (const u16*)x, x_stride, src, (const u16*)w, seg, n_experts, n_dim, k_dim, act);
+    const dim3 grid((unsigned)((n_dim + 127) / 128), (unsigned)tiles);
+    if (small)
+      grouped_linear_tiled_kernel<32, 128, 1, 4><<<grid, dim3(256), 0, s>>>((u16*)y, (const u16*)x, x_stride, src, (const u16*)w, seg,
+                                                                            n_experts, n_dim, k_dim, act);
+    else
+      grouped_linear_tiled_kernel<128, 128, 2, 2><<<grid, dim3(256), 0, s>>>((u16*)y, (const u16*)x, x_stride, src, (const u16*)w, seg,
+                                                                             n_experts, n_dim, k_dim, act);
     return hxm::check_launch();
   }
   const int64_t tiles = (max_rows + kGM - 1) / kGM + n_experts;

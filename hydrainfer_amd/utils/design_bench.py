@@ -320,18 +320,18 @@ def kezolix_kernel_table(size_name: str, dtype, dev, T: int = 4096, n_seqs: int 
     slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)], device=dev)
     seen = n_seqs * sum(i % chunk + 1 for i in range(q_len))
     us = _time_graph(lambda: ba.biased_attention(q, kc, vc, V, tok_seq, pos, q_cu, table, cu_b, 1 / math.sqrt(D), slopes, "chunk", chunk,
-                                                 max_q_len=q_len), dev, launches=2)
+                                                 max_q_len=q_len, max_kv_len=q_len), dev, launches=2)
     add(f"biased_attention, prefill {n_seqs} x {q_len} (chunks of {chunk}, head_dim {D})", us, flops=2 * H * (D + V) * seen)
     kcd, vcd = rnd(B * nbd, 16, G, D), rnd(B * nbd, 16, G, D)
     table_d, cu_bd = i32(torch.randperm(B * nbd)), i32(list(range(0, B * nbd + 1, nbd)))
     qd, seq_ids = rnd(B, H, D), i32(list(range(B)))
     keys = (ctx - 1) % chunk + 1
     us = _time_graph(lambda: ba.biased_attention(qd, kcd, vcd, V, seq_ids, posd, qcud, table_d, cu_bd, 1 / math.sqrt(D), slopes, "chunk",
-                                                 chunk, max_q_len=1), dev)
+                                                 chunk, max_q_len=1, max_kv_len=ctx), dev)
     add(f"biased_attention, decode {B} x {keys} keys of its chunk", us, 2 * B * keys * G * D * e + 2 * B * H * D * e)
     posd2 = i32([ctx - 1] * B)
     us = _time_graph(lambda: ba.biased_attention(qd, kcd, vcd, V, seq_ids, posd2, qcud, table_d, cu_bd, 1 / math.sqrt(D), slopes, "causal",
-                                                 0, max_q_len=1), dev)
+                                                 0, max_q_len=1, max_kv_len=ctx), dev)
     add(f"biased_attention, decode {B} x {ctx} keys (causal mask)", us, 2 * B * ctx * G * D * e + 2 * B * H * D * e)
     # experts
     logits, corr = f32(T, E + 1), f32(E) * 0.01

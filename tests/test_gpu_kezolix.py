@@ -220,12 +220,13 @@ def test_router_choice_bias_weights_and_ties(E, top):
     assert torch.equal(idx.cpu(), torch.arange(top, dtype=torch.int32).expand(4, top))
 
 
-@pytest.mark.parametrize("dims", [(38, 11, 3, 1), (96, 32, 5, 2), (128, 64, 70, 4)])
+@pytest.mark.parametrize("dims", [(38, 11, 3, 1, 77), (96, 32, 5, 2, 77), (128, 64, 70, 4, 77), (200, 72, 3, 2, 333)])
 def test_expert_plan_grouped_products_and_combine(dims):
+    """(the last case: hundreds of rows an expert — the large tiles of the bfloat16 product; sizes that are multiples of 8
+    but not of 32 or 64)"""
     from hydrainfer_amd._C.kernel.moe_mix import grouped_linear, moe_combine, moe_plan
-    W_, ff, E, top = dims
+    W_, ff, E, top, T = dims
     g = torch.Generator().manual_seed(ff)
-    T = 77
     h = torch.randn(T, W_, generator=g)
     up, down = torch.randn(E, ff, W_, generator=g) / math.sqrt(W_), torch.randn(E, W_, ff, generator=g) / math.sqrt(ff)
     idx = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).to(torch.int32)

@@ -74,7 +74,7 @@ def test_mix_library_header_and_binding_agree():
     from hydrainfer_amd import _lib
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     header = open(os.path.join(root, "include", "hydra_mix.h")).read()
-    declared = set(re.findall(r"^int (hxm_\w+)\(", header, flags=re.M))
+    declared = set(re.findall(r"^(?:int|int64_t) (hxm_\w+)\(", header, flags=re.M))
     assert declared == set(_lib._MIX_SIGNATURES)
     assert int(re.search(r"#define HXM_ABI_VERSION (\d+)", header).group(1)) == _lib.HXM_ABI_VERSION
 
