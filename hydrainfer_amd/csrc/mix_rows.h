@@ -42,4 +42,12 @@ __device__ __forceinline__ void block_sums(float (&v)[N], float* part) {
   for (int n = 0; n < N; ++n) v[n] = part[n] + part[N + n] + part[2 * N + n] + part[3 * N + n];
 }
 
+// A workgroup barrier that orders LDS traffic only: global loads and stores that are in flight (a prefetch for the next
+// step, results on their way out) are not waited for, as __syncthreads() would.  For exchanges through LDS alone.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 }  // namespace hx

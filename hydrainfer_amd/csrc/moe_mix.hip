@@ -3,7 +3,7 @@
 // and the weighted combine with an optional gated shared expert.  Nothing returns to the host between the router and the
 // combine: the products are launched for the most rows there can be and find their expert from the plan's segments.
 #include <cfloat>
-#include "hx_common.h"
+#include "mix_rows.h"
 #include "../../include/hydra_mix.h"
 
 namespace hxm {
@@ -261,7 +261,7 @@ __global__ __launch_bounds__(256) void grouped_linear_tiled_kernel(u16* __restri
     for (int p = 0; p < PA; ++p) *reinterpret_cast<u16x8*>(As + ((threadIdx.x + 256 * p) >> 3) * kLDK + ka[p]) = ra[p];
 #pragma unroll
     for (int p = 0; p < PB; ++p) *reinterpret_cast<u16x8*>(Bs + ((threadIdx.x + 256 * p) >> 3) * kLDK + kb[p]) = rb[p];
-    __syncthreads();
+    lds_barrier();      // (LDS only: the next slice's loads stay in flight)
     if (k0 + kKS < K) fetch(k0 + kKS);
 #pragma unroll
     for (int ks = 0; ks < kKS / 32; ++ks) {
@@ -277,7 +277,7 @@ __global__ __launch_bounds__(256) void grouped_linear_tiled_kernel(u16* __restri
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, af[i]), __builtin_bit_cast(bf16x8, bf[j]),
                                                               acc[i][j], 0, 0, 0);
     }
-    __syncthreads();
+    lds_barrier();      // (LDS only: the next slice's loads stay in flight)
   }
 #pragma unroll
   for (int i = 0; i < FM; ++i)
