@@ -109,6 +109,95 @@ __global__ __launch_bounds__(256) void depth_norm_kernel(hxm_depth_norm_args a) 
   }
 }
 
+// The same, four elements a lane at a time: width, y's stride and every pointer are multiples of four elements.
+__device__ __forceinline__ void row_stats4(const float* buf, float* part, int64_t W, float eps, int rms, float& shift, float& inv) {
+  const f32x4* b4 = reinterpret_cast<const f32x4*>(buf);
+  const int64_t n4 = W >> 2;
+  float mean = 0.f;
+  if (!rms) {
+    float s = 0.f;
+    for (int64_t i = threadIdx.x; i < n4; i += 256) {
+      const f32x4 v = b4[i];
+      s += (v[0] + v[1]) + (v[2] + v[3]);
+    }
+    mean = block_sum(s, part) / (float)W;
+  }
+  float ss = 0.f;
+  for (int64_t i = threadIdx.x; i < n4; i += 256) {
+    const f32x4 v = b4[i];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) ss += (v[k] - mean) * (v[k] - mean);
+  }
+  ss = block_sum(ss, part);
+  shift = mean;
+  inv = 1.0f / sqrtf(ss / (float)W + eps);
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void depth_norm_vec_kernel(hxm_depth_norm_args a) {
+  extern __shared__ float lds[];
+  f32x4* buf = reinterpret_cast<f32x4*>(lds);      // [W / 4]
+  float* part = lds + a.width;                      // [4]
+  typedef typename A::storage T;
+  const int64_t W = a.width, n4 = W >> 2, i_out = blockIdx.x;
+  const int64_t r = a.rows ? (int64_t)a.rows[i_out] : i_out;
+  const f32x4* xin = reinterpret_cast<const f32x4*>(a.x_in + r * W);
+  if (a.y) {
+    const T* y = (const T*)a.y + r * a.y_stride;
+    for (int64_t i = threadIdx.x; i < n4; i += 256) buf[i] = Row4<A>::load(y + 4 * i);
+    __syncthreads();
+    float shift, inv;
+    row_stats4(lds, part, W, a.eps, a.rms, shift, inv);
+    const f32x4* pw = reinterpret_cast<const f32x4*>(a.post_w);
+    for (int64_t i = threadIdx.x; i < n4; i += 256) {
+      const f32x4 v = buf[i], x = xin[i], w = pw[i];
+      f32x4 o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] = x[k] + a.mult * ((v[k] - shift) * inv * w[k]);
+      buf[i] = o;
+    }
+  } else {
+    for (int64_t i = threadIdx.x; i < n4; i += 256) buf[i] = xin[i];
+  }
+  // (every thread keeps to the elements i = tid + 256 k from here on: no barrier is needed until the next statistics)
+  if (a.level_out) {
+    f32x4* lo = reinterpret_cast<f32x4*>(a.level_out + r * W);
+    for (int64_t i = threadIdx.x; i < n4; i += 256) lo[i] = buf[i];
+  }
+  if (a.depth_w) {
+    for (int64_t i = threadIdx.x; i < n4; i += 256) {
+      f32x4 u = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < a.n_levels; ++j) {
+        const float* lv = a.levels + (int64_t)j * a.level_stride + r * W;
+        // the level written above is taken from LDS: the store to it need not have landed
+        const f32x4 v = (a.level_out && lv == a.level_out + r * W) ? buf[i] : reinterpret_cast<const f32x4*>(lv)[i];
+        const float w = a.depth_w[j];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) u[k] += w * v[k];
+      }
+      buf[i] = u;
+    }
+  }
+  if (a.x_out) {
+    f32x4* xo = reinterpret_cast<f32x4*>(a.x_out + i_out * W);
+    for (int64_t i = threadIdx.x; i < n4; i += 256) xo[i] = buf[i];
+  }
+  if (a.next_w) {
+    __syncthreads();
+    float shift, inv;
+    row_stats4(lds, part, W, a.eps, a.rms, shift, inv);
+    T* h = (T*)a.h_out + i_out * W;
+    const f32x4* nw = reinterpret_cast<const f32x4*>(a.next_w);
+    for (int64_t i = threadIdx.x; i < n4; i += 256) {
+      const f32x4 v = buf[i], w = nw[i];
+      f32x4 o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] = (v[k] - shift) * inv * w[k];
+      Row4<A>::store(h + 4 * i, o);
+    }
+  }
+}
+
 // vec: rows let a lane move four elements at a time (n, strides and pointers multiples of four elements)
 template <typename A>
 __global__ __launch_bounds__(256) void poly_norm_kernel(typename A::storage* __restrict__ out, int64_t out_stride,
@@ -208,9 +297,20 @@ extern "C" int hxm_depth_norm(const hxm_depth_norm_args* args, void* stream) {
   if (lds > 64 * 1024) return HX_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)a.n_out), block(256);
+  const uintptr_t es = a.dtype == HX_F32 ? 4 : 2;
+  auto by16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  const bool vec = a.width % 4 == 0 && by16(a.x_in) && by16(a.post_w) && by16(a.level_out) && by16(a.levels) && a.level_stride % 4 == 0 &&
+                   by16(a.x_out) && by16(a.next_w) && ((uintptr_t)a.y % (4 * es)) == 0 && a.y_stride % 4 == 0 &&
+                   ((uintptr_t)a.h_out % (4 * es)) == 0;
   switch (a.dtype) {
-    case HX_F32: depth_norm_kernel<F32><<<grid, block, lds, s>>>(a); break;
-    case HX_BF16: depth_norm_kernel<BF16><<<grid, block, lds, s>>>(a); break;
+    case HX_F32:
+      if (vec) depth_norm_vec_kernel<F32><<<grid, block, lds, s>>>(a);
+      else depth_norm_kernel<F32><<<grid, block, lds, s>>>(a);
+      break;
+    case HX_BF16:
+      if (vec) depth_norm_vec_kernel<BF16><<<grid, block, lds, s>>>(a);
+      else depth_norm_kernel<BF16><<<grid, block, lds, s>>>(a);
+      break;
     default: return HX_ERR_DTYPE;
   }
   return hxm::check_launch();

@@ -136,14 +136,14 @@ def _dev(t, dtype=torch.float32):
 
 
 # ------------------------------------------------------------------------------------------------ mechanisms alone
-@pytest.mark.parametrize("W_", [38, 96, 1024])
-def test_depth_norm_kernel_every_combination(W_):
+@pytest.mark.parametrize("W_,pad", [(38, 5), (96, 5), (96, 8), (1024, 8)])
+def test_depth_norm_kernel_every_combination(W_, pad):
     """The residual/norm kernel: pre-norm alone, a sublayer's result entering, a level written and averaged, selected rows,
-    RMS instead of layer norm."""
+    RMS instead of layer norm.  (pad 8: rows that a lane can move four elements at a time.)"""
     from hydrainfer_amd._C.kernel.depth_ops import depth_norm
     g = torch.Generator().manual_seed(W_)
     T, n_lv = 9, 4
-    x, y = torch.randn(T, W_, generator=g) * 3 + 1, torch.randn(T, W_ + 5, generator=g) * 2 - 0.5
+    x, y = torch.randn(T, W_, generator=g) * 3 + 1, torch.randn(T, W_ + pad, generator=g) * 2 - 0.5
     w1, w2 = torch.randn(W_, generator=g), torch.randn(W_, generator=g)
     levels = torch.randn(n_lv, T, W_, generator=g)
     dw = torch.randn(n_lv, generator=g)
