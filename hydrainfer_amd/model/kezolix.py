@@ -53,8 +53,9 @@ class MixerSpec:
     vdim: int                         # value size per head
     kv_heads: int = 0                 # attention: key / value heads (0: as many as heads)
     scale: float = 1.0                # attention
-    chunk: Optional[int] = None       # attention: size of the mask's chunks; None: every j <= i
+    chunk: Optional[int] = None       # attention: size of the mask's chunks (or of its window); None: every j <= i
     kv_from: Optional[int] = None     # attention: the layer whose keys and values this one reads
+    mask: str = "chunk"               # attention, with a size: "chunk" (i sees j <= i of its own chunk) | "window" (0 <= i - j < size)
 
     def __post_init__(self):
         if self.type == "attention":
@@ -136,9 +137,18 @@ class KezolixShape:
             m, kind = l["mixer"], l["type"]
             if kind == "attention":
                 mask = m.get("mask") or {}
+                mask_kind = str(mask.get("kind") or mask.get("type") or "chunk").lower()
+                if mask_kind in ("chunk", "chunked", "chunks", "block"):
+                    mask_kind = "chunk"
+                elif mask_kind in ("window", "sliding", "sliding_window", "local"):
+                    mask_kind = "window"
+                elif mask_kind in ("causal", "none", "full"):
+                    mask, mask_kind = {}, "chunk"
+                else:
+                    raise ValueError(f"layer {i}: unknown mask kind {mask_kind!r}")
                 mixer = MixerSpec(kind, int(m["heads"]), int(m["dim"]), int(m["vdim"]), int(m.get("kv_heads") or m["heads"]),
-                                  float(m["scale"]), int(mask["size"]) if mask.get("size") else None,
-                                  int(m["kv_from"]) if m.get("kv_from") is not None else None)
+                                  float(m.get("scale", 1.0)), int(mask["size"]) if mask.get("size") else None,
+                                  int(m["kv_from"]) if m.get("kv_from") is not None else None, mask_kind)
             elif kind == "hgrn2":
                 mixer = MixerSpec(kind, int(m["heads"]), int(m["dim"]), int(m["vdim"]))
             else:
@@ -166,7 +176,7 @@ class KezolixShape:
             if m.type == "attention":
                 mixer.update({"kv_heads": m.kv_heads, "scale": m.scale})
                 if m.chunk:
-                    mixer["mask"] = {"size": m.chunk}
+                    mixer["mask"] = {"size": m.chunk} if m.mask == "chunk" else {"kind": m.mask, "size": m.chunk}
                 if m.kv_from is not None:
                     mixer["kv_from"] = m.kv_from
             mlp = None
@@ -366,7 +376,7 @@ class KezolixForCausalLM:
         else:
             q = qk_norm_cache(proj, H * D, 0, 0, w.q_norm, None, sh.norm_eps, G)
         o = biased_attention(q.view(T, H, D), kc, vc, V, seq.tok_seq, position_ids, ap.q_cu_seq_lens, ap.block_tables,
-                             ap.cu_blocks_lens, m.scale, w.slopes, "chunk" if m.chunk else "causal", m.chunk or 0,
+                             ap.cu_blocks_lens, m.scale, w.slopes, m.mask if m.chunk else "causal", m.chunk or 0,
                              max_q_len=ap.q_max_seq_len, kv_heads=G, max_kv_len=ap.kv_max_seq_len)
         return torch.matmul(o.view(T, H * V), w.o.t())
 

@@ -26,11 +26,14 @@ def head_slopes(n_heads: int) -> torch.Tensor:
     return torch.tensor([2.0 ** (-8.0 * (h + 1) / n_heads) for h in range(n_heads)], dtype=F)
 
 
-def visible(n: int, chunk: Optional[int]) -> torch.Tensor:
-    """[n, n] bool: query i sees key j iff j <= i and, with chunks, both lie in the same chunk counted from 0."""
+def visible(n: int, chunk: Optional[int], kind: str = "chunk") -> torch.Tensor:
+    """[n, n] bool: query i sees key j iff j <= i and, with chunks, both lie in the same chunk counted from 0 (kind
+    "window": i - j < size instead)."""
     i, j = torch.arange(n)[:, None], torch.arange(n)[None, :]
     ok = j <= i
-    if chunk:
+    if chunk and kind == "window":
+        ok &= i - j < chunk
+    elif chunk:
         ok &= (i // chunk) == (j // chunk)
     return ok
 
@@ -49,7 +52,7 @@ def attention(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m: dict, eps:
     G = m.get("kv_heads", H)
     q = (rms_div(h @ W[p + "q"].T, eps) * W[p + "q.norm"]).reshape(n, H, D)
     k, v = k.reshape(n, G, D), v.reshape(n, G, V)
-    see = visible(n, (m.get("mask") or {}).get("size"))
+    see = visible(n, (m.get("mask") or {}).get("size"), (m.get("mask") or {}).get("kind", "chunk"))
     dist = (torch.arange(n)[:, None] - torch.arange(n)[None, :]).to(F)
     slopes = head_slopes(H)
     out = torch.zeros(n, H, V, dtype=F)

@@ -37,7 +37,8 @@ def _shape(kind: str):
                                      L(rec(3, 16, 40), moe(32, 5, 2, 1.7, 48)),
                                      L(att(6, 16, 24, 2, 0.2, 7, kv_from=0), None),
                                      L(rec(1, 24, 72), moe(64, 9, 3, 0.8, None)),
-                                     L(att(2, 32, 8, 1, 0.25, None), F("dense", 40))],
+                                     L(att(2, 32, 8, 1, 0.25, None), F("dense", 40)),
+                                     L(att(4, 8, 16, 2, 0.35, 9, mask="window"), None)],      # (a sliding window: the kernel's third mask)
                             max_position_embeddings=256, norm_eps=1e-5, residual_mult=0.4)
     if kind == "odd":         # nothing a multiple of four or of sixteen: every kernel's element-by-element path; top 1
         return KezolixShape(45, 38, [L(rec(3, 6, 10), F("dense", 26)),
@@ -485,8 +486,8 @@ def test_specs_the_engine_reads():
     a, r, h = (_model(_shape(k), _weights(_shape(k)), torch.float32).language_model for k in ("attention", "recurrent", "hybrid"))
     assert a.state_spec() is None and a.cache_spec() == {"n_layers": 2, "n_tokens": 2, "n_heads": 4, "head_size": 64}
     assert r.state_spec() == {"rows": 3, "width": 2 * 64 * 128} and r.cache_spec()["n_layers"] == 1
-    assert h.cache_spec() == {"n_layers": 2, "n_tokens": 2, "n_heads": 2, "head_size": 32}      # the borrower has no plane
-    assert h.shape.cache_plane == {0: 0, 2: 0, 4: 1} and h.shape.state_row == {1: 0, 3: 1}
+    assert h.cache_spec() == {"n_layers": 3, "n_tokens": 2, "n_heads": 2, "head_size": 32}      # the borrower has no plane
+    assert h.shape.cache_plane == {0: 0, 2: 0, 4: 1, 5: 2} and h.shape.state_row == {1: 0, 3: 1}
 
 
 @pytest.mark.parametrize("kind", ["hybrid", "odd", "recurrent"])

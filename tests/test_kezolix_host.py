@@ -31,6 +31,10 @@ def test_shape_from_config_planes_rows_and_names():
     assert sh.layers[2].mixer.chunk is None and sh.layers[4].mixer.chunk == 4 and sh.layers[2].mlp is None
     assert sh.layers[3].mlp.shared_ff is None and sh.layers[1].mlp.shared_ff == 24 and sh.layers[1].mlp.router_scale == 1.25
     assert KezolixShape.from_config(sh.to_config()).to_config() == sh.to_config()
+    w = _config()
+    w["layers"][2]["mixer"]["mask"] = {"kind": "window", "size": 6}
+    ws = KezolixShape.from_config(w)
+    assert (ws.layers[2].mixer.mask, ws.layers[2].mixer.chunk) == ("window", 6) and ws.to_config()["layers"][2]["mixer"]["mask"] == {"kind": "window", "size": 6}
     names = tensor_shapes(sh)
     assert names["l1.mix.k"] == (16, 24) and names["l1.mix.k.norm"] == (16,) and names["l1.mix.q.norm"] == (48,)
     assert "l4.mix.k" not in names and "l4.mix.v" not in names and names["l4.mix.o"] == (24, 72)
