@@ -12,9 +12,10 @@ from hydrainfer_amd._C.kernel.stream_ops import SequenceState
 
 def gated_recurrence(q_pre: Tensor, f_pre: Tensor, v: Tensor, f_bias: Tensor, low: Tensor, norm_w: Tensor, eps: float,
                      seq: SequenceState, state_row: int, q_cu: Tensor, positions: Tensor, heads: int, dim: int,
-                     vdim: int) -> Tensor:
+                     vdim: int, max_q_len: int = 0) -> Tensor:
     """q_pre, f_pre: [n_tokens, heads * dim]; v: [n_tokens, heads * vdim] (views of one projection will do: contiguous rows).
     seq.state: float32 [n_slots, n_rows, >= heads * dim * vdim]; this layer's state is row `state_row` of a slot.
+    max_q_len: the longest portion of the batch when known (1: every sequence brings one token — a decode step's kernel).
     Returns [n_tokens, heads * vdim] in the inputs' dtype."""
     _lib.require_gpu(q_pre, f_pre, v, f_bias, low, norm_w, seq.state, seq.slots, q_cu, positions)
     T = q_pre.shape[0]
@@ -42,6 +43,6 @@ def gated_recurrence(q_pre: Tensor, f_pre: Tensor, v: Tensor, f_bias: Tensor, lo
     _lib.mix_check(_lib.mix_lib().hxm_gated_recurrence(
         out.data_ptr(), q_pre.data_ptr(), q_pre.stride(0), f_pre.data_ptr(), f_pre.stride(0), v.data_ptr(), v.stride(0),
         f_bias.data_ptr(), low.data_ptr(), norm_w.data_ptr(), float(eps), base, st.stride(0), q_cu.data_ptr(),
-        positions.data_ptr(), seq.slots.data_ptr(), n_seq, T, int(heads), int(dim), int(vdim), ws.data_ptr(), n_ws,
+        positions.data_ptr(), seq.slots.data_ptr(), n_seq, T, int(heads), int(dim), int(vdim), int(max_q_len), ws.data_ptr(), n_ws,
         _lib._DTYPE[dt], _lib.current_stream()), "gated_recurrence")
     return out

@@ -281,7 +281,7 @@ _MIX_SIGNATURES = {
     "hxm_gated_recurrence_workspace": (c_int64, [c_int64, c_int32, c_int32, c_int32]),
     "hxm_gated_recurrence": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                      c_float, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32,
-                                     c_int32, c_void_p, c_int64, c_int, c_void_p]),
+                                     c_int32, c_int32, c_void_p, c_int64, c_int, c_void_p]),
     "hxm_qk_norm_cache": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                   c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int64, c_int,
                                   c_void_p]),

@@ -40,14 +40,15 @@ struct RecArgs {
   const int32_t* slots;
   float* ws;                     // [n_parts][n_tokens][heads * vdim]
   int64_t n_tokens;
-  int32_t heads, dim, vdim, n_cw, n_parts, n_waves;
+  int32_t heads, dim, vdim, n_cw, n_parts, n_waves, max_q_len;
   float eps;
 };
 
 template <typename A, int DR>
 __global__ __launch_bounds__(64 * kMaxWaves) void gated_recurrence_scan_kernel(RecArgs a) {
   __shared__ __attribute__((aligned(16))) float gates[kTC * kMaxWaves * DR * 2];      // [token][row of the part][f, silu(q)]
-  __shared__ float po[kTC * kMaxWaves * 64];                                           // [token][wave][lane]
+  __shared__ __attribute__((aligned(16))) float po[kTC * kMaxWaves * 64];              // [token][wave][lane]
+  __shared__ float vs[kTC * 64];                                                       // [token][lane]: the chunk's values
   typedef typename A::storage T;
   const int seq = blockIdx.x, head = blockIdx.y;
   const int cw = blockIdx.z % a.n_cw, part = blockIdx.z / a.n_cw;
@@ -75,10 +76,11 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gated_recurrence_scan_kernel(R
   const float* lw = a.low + head * D;
   float* wo = a.ws + (int64_t)part * a.n_tokens * (a.heads * V) + head * V;
   const int n_threads = NW * 64;
+  const bool pair_ok = (V & 1) == 0 && (((uintptr_t)a.ws) & 7) == 0;      // two floats of the workspace at a time
   // the pre-activations a thread turns into gates (element e of a chunk: token e / rows_part, row e % rows_part) and the
   // lane's values, asked for one chunk ahead
   constexpr int EPT = kTC * DR / 64;
-  float qn[EPT], fn[EPT], vn[kTC];
+  float qn[EPT], fn[EPT];
   auto fetch = [&](int t0) __attribute__((always_inline)) {
     const int nt = t_end - t0 < kTC ? t_end - t0 : kTC;
 #pragma unroll
@@ -89,16 +91,31 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gated_recurrence_scan_kernel(R
       qn[e] = ok ? A::to_float(qp[(int64_t)(t0 + tt) * a.q_stride + d]) : 0.f;
       fn[e] = ok ? A::to_float(fp[(int64_t)(t0 + tt) * a.f_stride + d]) : 0.f;
     }
+  };
+  // The chunk's values [token][column of this group]: every wave of the workgroup needs the same 16 x 64, so the workgroup
+  // brings them once (a few loads a thread, one chunk ahead) and hands them round through LDS — one load a lane and
+  // token in every wave was the largest single cost of this kernel (vector memory instructions, not bytes).
+  float vn[kTC];      // (kTC values a thread when the workgroup is a single wave, two when it has eight)
+  auto fetch_v = [&](int t0) __attribute__((always_inline)) {
+    const int nt = t_end - t0 < kTC ? t_end - t0 : kTC;
 #pragma unroll
-    for (int tt = 0; tt < kTC; ++tt)
-      vn[tt] = (col_ok && tt < nt) ? A::to_float(vp[(int64_t)(t0 + tt) * a.v_stride + col]) : 0.f;
+    for (int k = 0; k < kTC; ++k) {
+      const int i = threadIdx.x + k * n_threads;      // token i / 64, column i % 64
+      if (i < kTC * 64) {
+        const int tt = i >> 6, c = cw * 64 + (i & 63);
+        vn[k] = (tt < nt && c < V) ? A::to_float(vp[(int64_t)(t0 + tt) * a.v_stride + c]) : 0.f;
+      }
+    }
   };
   fetch(t_begin);
+  fetch_v(t_begin);
   for (int t0 = t_begin; t0 < t_end; t0 += kTC) {
     const int nt = t_end - t0 < kTC ? t_end - t0 : kTC;
-    float vv[kTC];
 #pragma unroll
-    for (int tt = 0; tt < kTC; ++tt) vv[tt] = vn[tt];
+    for (int k = 0; k < kTC; ++k) {
+      const int i = threadIdx.x + k * n_threads;
+      if (i < kTC * 64) vs[i] = vn[k];
+    }
 #pragma unroll
     for (int e = 0; e < EPT; ++e) {
       const int i = threadIdx.x + e * n_threads;
@@ -112,8 +129,14 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gated_recurrence_scan_kernel(R
       gates[2 * i] = f;
       gates[2 * i + 1] = q;
     }
-    if (t0 + kTC < t_end) fetch(t0 + kTC);
+    if (t0 + kTC < t_end) {
+      fetch(t0 + kTC);
+      fetch_v(t0 + kTC);
+    }
     __syncthreads();
+    float vv[kTC];
+#pragma unroll
+    for (int tt = 0; tt < kTC; ++tt) vv[tt] = vs[tt * 64 + lane];
 #pragma unroll
     for (int tt = 0; tt < kTC; ++tt) {
       if (tt < nt) {
@@ -132,13 +155,20 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gated_recurrence_scan_kernel(R
       }
     }
     __syncthreads();
-    // the waves' partial o's of the chunk, summed: thread (tt, lane) pairs dealt over the workgroup
-    for (int i = threadIdx.x; i < nt * 64; i += n_threads) {
-      const int tt = i >> 6, ln = i & 63, c = cw * 64 + ln;
-      if (c < V) {
-        float o = 0.f;
-        for (int w = 0; w < NW; ++w) o += po[(tt * kMaxWaves + w) * 64 + ln];
-        wo[(int64_t)(t0 + tt) * (a.heads * V) + c] = o;
+    // the waves' partial o's of the chunk, summed: (token, pair of columns) dealt over the workgroup
+    for (int i = threadIdx.x; i < nt * 32; i += n_threads) {
+      const int tt = i >> 5, ln = (i & 31) * 2, c = cw * 64 + ln;
+      float o0 = 0.f, o1 = 0.f;
+      for (int w = 0; w < NW; ++w) {
+        const float2 p2 = *reinterpret_cast<const float2*>(po + (tt * kMaxWaves + w) * 64 + ln);
+        o0 += p2.x;
+        o1 += p2.y;
+      }
+      float* dst = wo + (int64_t)(t0 + tt) * (a.heads * V) + c;
+      if (c + 1 < V && pair_ok) *reinterpret_cast<float2*>(dst) = float2{o0, o1};
+      else {
+        if (c < V) dst[0] = o0;
+        if (c + 1 < V) dst[1] = o1;
       }
     }
     // (the next chunk's gates are written while slow waves may still sum: they read po only; po is written again after
@@ -148,6 +178,57 @@ __global__ __launch_bounds__(64 * kMaxWaves) void gated_recurrence_scan_kernel(R
   for (int r = 0; r < DR; ++r) {
     const int d = d0 + r;
     if (col_ok && d < D) slot[(int64_t)d * V + col] = S[r];
+  }
+}
+
+// The same for batches in which every sequence brings ONE token (decode steps): no chunks, no staging — a wave reads its
+// rows of the state, lanes 0 .. DR - 1 work out the rows' gates and hand them round with v_readlane, the state goes back.
+template <typename A, int DR>
+__global__ __launch_bounds__(64 * kMaxWaves) void gated_recurrence_step_kernel(RecArgs a) {
+  __shared__ float po[kMaxWaves * 64];
+  typedef typename A::storage T;
+  const int seq = blockIdx.x, head = blockIdx.y;
+  const int cw = blockIdx.z % a.n_cw, part = blockIdx.z / a.n_cw;
+  const int D = a.dim, V = a.vdim, NW = a.n_waves;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int col = cw * 64 + lane;
+  const bool col_ok = col < V;
+  const int d0 = (part * NW + wave) * DR;
+  const int t = a.q_cu[seq];
+  if (a.q_cu[seq + 1] <= t) return;
+  float* slot = a.state + (int64_t)a.slots[seq] * a.slot_stride + (int64_t)head * D * V;
+  const bool fresh = a.positions[t] == 0;
+  float S[DR];
+#pragma unroll
+  for (int r = 0; r < DR; ++r) {
+    const int d = d0 + r;
+    S[r] = (!fresh && col_ok && d < D) ? slot[(int64_t)d * V + col] : 0.f;
+  }
+  float f = 1.f, q = 0.f;      // lane r < DR: row d0 + r (past D: the state stays, nothing is read out)
+  if (lane < DR && d0 + lane < D) {
+    const int hd = head * D + d0 + lane;
+    const float qv = A::to_float(((const T*)a.q_pre)[(int64_t)t * a.q_stride + hd]);
+    const float fv = A::to_float(((const T*)a.f_pre)[(int64_t)t * a.f_stride + hd]) + a.f_bias[hd];
+    const float l = a.low[hd];
+    q = qv / (1.0f + expf(-qv));
+    f = l + (1.0f - l) / (1.0f + expf(-fv));
+  }
+  const float v = col_ok ? A::to_float(((const T*)a.v)[(int64_t)t * a.v_stride + head * V + col]) : 0.f;
+  float o = 0.f;
+#pragma unroll
+  for (int r = 0; r < DR; ++r) {
+    const float fr = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), r));
+    const float qr = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(q), r));
+    S[r] = v + fr * (S[r] - v);
+    o += qr * S[r];
+    if (col_ok && d0 + r < D) slot[(int64_t)(d0 + r) * V + col] = S[r];
+  }
+  po[wave * 64 + lane] = o;
+  __syncthreads();
+  if (wave == 0 && col_ok) {
+    float sum = 0.f;
+    for (int w = 0; w < NW; ++w) sum += po[w * 64 + lane];
+    a.ws[(int64_t)part * a.n_tokens * (a.heads * V) + (int64_t)t * (a.heads * V) + head * V + col] = sum;
   }
 }
 
@@ -191,9 +272,12 @@ void recurrence_layout(int dim, int& dr, int& n_waves, int& n_parts) {
 template <typename A>
 int launch_recurrence(const RecArgs& a, int n_seq, int dr, hipStream_t s) {
   const dim3 grid((unsigned)n_seq, (unsigned)a.heads, (unsigned)(a.n_cw * a.n_parts)), block((unsigned)(a.n_waves * 64));
-  switch (dr) {
-    case 4: gated_recurrence_scan_kernel<A, 4><<<grid, block, 0, s>>>(a); break;
-    default: gated_recurrence_scan_kernel<A, 8><<<grid, block, 0, s>>>(a); break;
+  if (a.max_q_len == 1) {
+    if (dr == 4) gated_recurrence_step_kernel<A, 4><<<grid, block, 0, s>>>(a);
+    else gated_recurrence_step_kernel<A, 8><<<grid, block, 0, s>>>(a);
+  } else {
+    if (dr == 4) gated_recurrence_scan_kernel<A, 4><<<grid, block, 0, s>>>(a);
+    else gated_recurrence_scan_kernel<A, 8><<<grid, block, 0, s>>>(a);
   }
   gated_recurrence_norm_kernel<A><<<dim3((unsigned)((a.n_tokens * a.heads + 3) / 4)), dim3(256), 0, s>>>(a);
   return hxm::check_launch();
@@ -212,8 +296,8 @@ extern "C" int hxm_gated_recurrence(void* out, const void* q_pre, int64_t q_stri
                                     const void* v, int64_t v_stride, const float* f_bias, const float* low,
                                     const float* norm_w, float eps, float* state, int64_t slot_stride, const int32_t* q_cu,
                                     const int32_t* positions, const int32_t* slots, int32_t n_seq, int64_t n_tokens,
-                                    int32_t heads, int32_t dim, int32_t vdim, float* ws, int64_t ws_floats, int dtype,
-                                    void* stream) {
+                                    int32_t heads, int32_t dim, int32_t vdim, int32_t max_q_len, float* ws,
+                                    int64_t ws_floats, int dtype, void* stream) {
   if (n_seq < 0 || n_tokens < 0 || heads < 1 || dim < 1 || vdim < 1 || vdim > 1024 || heads > 65535) return HX_ERR_SHAPE;
   if (n_seq == 0 || n_tokens == 0) return HX_OK;
   if (!out || !q_pre || !f_pre || !v || !f_bias || !low || !norm_w || !state || !q_cu || !positions || !slots || !ws) return HX_ERR_NULL;
@@ -223,7 +307,7 @@ extern "C" int hxm_gated_recurrence(void* out, const void* q_pre, int64_t q_stri
   a.q_stride = q_stride; a.f_stride = f_stride; a.v_stride = v_stride;
   a.f_bias = f_bias; a.low = low; a.norm_w = norm_w; a.state = state; a.slot_stride = slot_stride;
   a.q_cu = q_cu; a.positions = positions; a.slots = slots; a.ws = ws; a.n_tokens = n_tokens;
-  a.heads = heads; a.dim = dim; a.vdim = vdim; a.eps = eps;
+  a.heads = heads; a.dim = dim; a.vdim = vdim; a.eps = eps; a.max_q_len = max_q_len;
   a.n_cw = (vdim + 63) / 64;
   int dr;
   recurrence_layout(dim, dr, a.n_waves, a.n_parts);

@@ -385,7 +385,8 @@ class KezolixForCausalLM:
         HD = m.heads * m.dim
         proj = torch.matmul(h, w.w_in.t())                           # [T, q | f | v]
         o = gated_recurrence(proj[:, :HD], proj[:, HD:2 * HD], proj[:, 2 * HD:], w.f_bias, w.low, w.o_norm, sh.norm_eps, seq,
-                             sh.state_row[i], params.attention_params[0].q_cu_seq_lens, position_ids, m.heads, m.dim, m.vdim)
+                             sh.state_row[i], params.attention_params[0].q_cu_seq_lens, position_ids, m.heads, m.dim, m.vdim,
+                             max_q_len=params.attention_params[0].q_max_seq_len)
         return torch.matmul(o, w.o.t())
 
     def _feed_forward(self, i: int, h: Tensor) -> Tensor:

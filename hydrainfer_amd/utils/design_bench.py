@@ -306,7 +306,7 @@ def kezolix_kernel_table(size_name: str, dtype, dev, T: int = 4096, n_seqs: int 
     posd, qcud = i32([ctx - 1] * B), i32(list(range(B + 1)))
     seqd = SequenceState(state, i32(list(range(B))), i32(list(range(B))))
     us = _time_graph(lambda: gated_recurrence(proj[:B, :H * D], proj[:B, H * D:2 * H * D], proj[:B, 2 * H * D:], fb, low, nw, 1e-5, seqd,
-                                              0, qcud, posd, H, D, V), dev)
+                                              0, qcud, posd, H, D, V, max_q_len=1), dev)
     add(f"gated_recurrence, decode {B} sequences (state read and written)", us, 2 * B * H * D * V * 4)
     # attention
     nb, nbd = (q_len + 15) // 16, (ctx + 15) // 16

@@ -196,13 +196,15 @@ int hxm_moe_combine(void* out, const void* y, const int32_t* row_of, const float
  * state: float, slot s at state + s * slot_stride, [heads, dim, vdim] contiguous within a slot.  A sequence whose portion
  * starts at position 0 starts from a zero state (the slot is not read); the slot receives the state after the portion's
  * last token.  q_cu: int32 [n_seq + 1]; positions: int32 [n_tokens]; slots: int32 [n_seq].  ws: float workspace of at least
- * hxm_gated_recurrence_workspace(n_tokens, heads, dim, vdim) floats (the partial results of the key channels' parts). */
+ * hxm_gated_recurrence_workspace(n_tokens, heads, dim, vdim) floats (the partial results of the key channels' parts).
+ * max_q_len: the longest portion of the batch if the caller knows it, else 0; 1 (every sequence brings one token) takes a
+ * kernel without the chunk machinery. */
 int64_t hxm_gated_recurrence_workspace(int64_t n_tokens, int32_t heads, int32_t dim, int32_t vdim);
 int hxm_gated_recurrence(void* out, const void* q_pre, int64_t q_stride, const void* f_pre, int64_t f_stride, const void* v,
                          int64_t v_stride, const float* f_bias, const float* low, const float* norm_w, float eps,
                          float* state, int64_t slot_stride, const int32_t* q_cu, const int32_t* positions,
                          const int32_t* slots, int32_t n_seq, int64_t n_tokens, int32_t heads, int32_t dim, int32_t vdim,
-                         float* ws, int64_t ws_floats, int dtype, void* stream);
+                         int32_t max_q_len, float* ws, int64_t ws_floats, int dtype, void* stream);
 
 /* ------------------------------------------------------------------------------------------------------------------
  * Grouped-query attention over a paged key/value cache with a linear distance bias and a mask.

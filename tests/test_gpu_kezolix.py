@@ -313,6 +313,20 @@ def test_recurrence_kernel_portions_slots_and_fresh_starts(H, D, V):
         got_a = torch.cat([o1[:16], o2[:2], o3])
         got_c = torch.cat([o1[17:], o2[2:]])
         _close(got_a, refs[0][0], tol, "first sequence in three portions")
+        # single tokens through the decode step's kernel: the second sequence from a stale slot, then one more token of it
+        more = torch.randn(1, 2 * H * D + H * V, generator=g).to(dtype)
+        two, _ = ref_of(torch.cat([pq[1], more]).float())
+        P = _dev(torch.cat([pq[1], c[:1]]), dtype)
+        seq = SequenceState(state, torch.tensor([1, 2], dtype=torch.int32, device=DEV), None)
+        step = lambda rows, pos0, sl: gated_recurrence(
+            rows[:, :H * D], rows[:, H * D:2 * H * D], rows[:, 2 * H * D:], _dev(Wd["f.b"]), _dev(Wd["lower"]), _dev(Wd["norm"]), eps,
+            SequenceState(state, torch.tensor(sl, dtype=torch.int32, device=DEV), None), 1,
+            torch.arange(len(sl) + 1, dtype=torch.int32, device=DEV), torch.tensor(pos0, dtype=torch.int32, device=DEV), H, D, V, max_q_len=1)
+        o = step(P, [0, 0], [1, 2])
+        _close(o[:1], two[:1], tol, "decode step from position 0")
+        _close(o[1:], refs[2][0][:1], tol, "decode step, second sequence of the batch")
+        o = step(_dev(more, dtype), [1], [1])
+        _close(o, two[1:], tol, "decode step from the slot")
         _close(got_c, refs[2][0], tol, "third sequence in two portions")
 
 
