@@ -316,19 +316,13 @@ __global__ __launch_bounds__(256) void biased_attn_tile_kernel(hxm_biased_attn_a
         p[s] = seen ? sc[s][i] * a.scale - slope[i] * (float)(pos[i] - key) : -INFINITY;
         mx = fmaxf(mx, p[s]);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 4, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 8, 64));
+      mx = row16_max(mx);      // (the sixteen lanes that hold the row's scores: one DPP row)
       const float m_new = fmaxf(m[i], mx);
       const float corr = __expf(m[i] - m_new);
       p[0] = __expf(p[0] - m_new);       // exp(-inf) = 0 for a key the row does not see
       p[1] = __expf(p[1] - m_new);
       float ps = p[0] + p[1];
-      ps += __shfl_xor(ps, 1, 64);
-      ps += __shfl_xor(ps, 2, 64);
-      ps += __shfl_xor(ps, 4, 64);
-      ps += __shfl_xor(ps, 8, 64);
+      ps = row16_sum(ps);
       l[i] = l[i] * corr + ps;
       m[i] = m_new;
 #pragma unroll

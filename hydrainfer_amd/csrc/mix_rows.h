@@ -42,6 +42,31 @@ __device__ __forceinline__ void block_sums(float (&v)[N], float* part) {
   for (int n = 0; n < N; ++n) v[n] = part[n] + part[N + n] + part[2 * N + n] + part[3 * N + n];
 }
 
+// Reductions over the 16 lanes of a DPP row (lanes 16 k .. 16 k + 15) on the vector ALU alone — a shuffle goes through
+// the LDS crossbar (ds_bpermute) and waits for it.  Every lane ends with the row's result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+constexpr int kDppXor1 = 0xB1;          // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;          // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;   // lanes of each half of the row in reverse order
+constexpr int kDppMirror = 0x140;       // the row in reverse order
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_move<kDppXor1>(v);
+  v += dpp_move<kDppXor2>(v);
+  v += dpp_move<kDppHalfMirror>(v);
+  v += dpp_move<kDppMirror>(v);
+  return v;
+}
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_move<kDppXor1>(v));
+  v = fmaxf(v, dpp_move<kDppXor2>(v));
+  v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+  v = fmaxf(v, dpp_move<kDppMirror>(v));
+  return v;
+}
+
 // A workgroup barrier that orders LDS traffic only: global loads and stores that are in flight (a prefetch for the next
 // step, results on their way out) are not waited for, as __syncthreads() would.  For exchanges through LDS alone.
 __device__ __forceinline__ void lds_barrier() {
