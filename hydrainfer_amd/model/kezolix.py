@@ -42,7 +42,6 @@ from hydrainfer_amd._C.kernel.stream_ops import SequenceState
 
 ARCHITECTURE = "Kezolix"
 SLOPE_EXPONENT = 8.0          # slope_h = 2^(-SLOPE_EXPONENT (h + 1) / H)
-ROUTER_WEIGHT_FLOOR = 1e-20   # (added to the sum of the chosen scores inside the router kernel)
 
 
 @dataclass

@@ -201,7 +201,7 @@ def test_embedding_poly_norm_and_squared_relu_kernels():
             _close(out, torch.relu(zq[:, :n].double()) ** 2, tol, "squared ReLU")
 
 
-@pytest.mark.parametrize("E,top", [(5, 2), (12, 4), (70, 1), (200, 8), (9, 9)])
+@pytest.mark.parametrize("E,top", [(5, 2), (11, 4), (70, 1), (200, 8), (9, 9)])
 def test_router_choice_bias_weights_and_ties(E, top):
     from hydrainfer_amd._C.kernel.moe_mix import route_softmax_topk
     g = torch.Generator().manual_seed(E)
@@ -263,7 +263,7 @@ def test_expert_plan_grouped_products_and_combine(dims):
         _close(out, ref - torch.sigmoid(gate[:, 1:2].double()) * sq.double(), tol, "without a shared expert")
 
 
-@pytest.mark.parametrize("H,D,V", [(2, 32, 64), (3, 6, 10), (1, 130, 32), (2, 64, 128), (1, 24, 200)])
+@pytest.mark.parametrize("H,D,V", [(3, 16, 64), (3, 6, 10), (1, 130, 32), (2, 64, 128), (1, 24, 200)])
 def test_recurrence_kernel_portions_slots_and_fresh_starts(H, D, V):
     """Whole sequences, then the same cut into portions through state slots that held other sequences before."""
     from hydrainfer_amd._C.kernel.recurrence import gated_recurrence
@@ -349,7 +349,7 @@ def _paged(rows_k, rows_v, block_size, G, head_size, seed, dtype):
     return kc.to(DEV), vc.to(DEV), torch.tensor(table, dtype=torch.int32, device=DEV), torch.tensor(cu, dtype=torch.int32, device=DEV)
 
 
-@pytest.mark.parametrize("H,G,D,V,mask,size", [(4, 2, 64, 48, "chunk", 24), (3, 3, 5, 7, "chunk", 5), (6, 1, 16, 130, "causal", 0),
+@pytest.mark.parametrize("H,G,D,V,mask,size", [(4, 2, 64, 40, "chunk", 24), (3, 3, 5, 7, "chunk", 5), (6, 1, 16, 130, "causal", 0),
                                               (2, 2, 32, 32, "window", 17), (8, 2, 128, 64, "chunk", 100)])
 def test_attention_kernel_edges_far_keys_and_page_borders(H, G, D, V, mask, size):
     """One key made to stand out (query and key scaled so that its score dominates): far back, just inside and just outside
