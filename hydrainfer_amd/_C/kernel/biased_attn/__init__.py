@@ -67,7 +67,9 @@ def biased_attention(q: Tensor, key_cache: Tensor, value_cache: Tensor, vdim: in
     """q: [n_tokens, n_heads, dim] contiguous.  kv_heads: the key / value heads in use (the first of every cache row;
     default: all the plane has).  max_q_len: the longest portion of the batch; max_kv_len: the most keys a sequence holds —
     with few rows in the launch (decode steps) the keys of every tile are dealt to several waves.  form: "auto" (bfloat16
-    with sizes that are multiples of 8: the MFMA tile form) or "rows" (one wave per token and head, any dtype and size).
+    with sizes that are multiples of 8: the MFMA forms — portions of prompts share every chunk of keys between four row
+    tiles, decode steps split the keys), "tile" (the MFMA tile form throughout) or "rows" (one wave per token and head, any
+    dtype and size).
     Returns [n_tokens, n_heads, vdim]."""
     _lib.require_gpu(q, key_cache, value_cache, tok_seq, positions, q_cu, block_table, cu_block_lens, slopes)
     if q.dim() != 3 or not q.is_contiguous() or key_cache.dtype != q.dtype or value_cache.dtype != q.dtype:
@@ -98,8 +100,8 @@ def biased_attention(q: Tensor, key_cache: Tensor, value_cache: Tensor, vdim: in
     a.n_tokens, a.n_heads, a.kv_heads, a.dim, a.vdim = T, H, G, D, int(vdim)
     a.mask_kind, a.mask_size, a.scale, a.dtype = MASK_KINDS[mask], int(mask_size), float(scale), _code(q.dtype)
     a.n_seq, a.max_q_len = n_seq, int(max_q_len)
-    a.form, a.n_splits, a.ws_o, a.ws_ml = {"auto": 0, "rows": 1}[form], 1, None, None
-    if form == "auto" and q.dtype == torch.bfloat16 and max_q_len > 0 and max_kv_len > 0 and D % 8 == 0 and vdim % 8 == 0 \
+    a.form, a.n_splits, a.ws_o, a.ws_ml = {"auto": 0, "rows": 1, "tile": 2}[form], 1, None, None
+    if form in ("auto", "tile") and q.dtype == torch.bfloat16 and max_q_len > 0 and max_kv_len > 0 and D % 8 == 0 and vdim % 8 == 0 \
             and D <= 256 and vdim <= 256:
         # key splits: enough waves to fill the chip when the launch has few row tiles, at least two 32-key chunks a split
         tiles = n_seq * G * ((max_q_len * (H // G) + 15) // 16)

@@ -387,6 +387,188 @@ __global__ __launch_bounds__(256) void biased_attn_tile_kernel(hxm_biased_attn_a
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Group form (bfloat16, portions of prompts, head sizes up to 128): a workgroup of four waves takes four consecutive row
+// tiles (64 rows) of ONE (sequence, key head) and ONE image of every 32-key chunk.  The tile form is bound by its loads —
+// sixteen 16-byte load instructions per chunk and wave, each touching sixteen half cache lines; here the workgroup brings
+// a chunk's key and value rows once, in whole rows (two to four loads a thread), into one of two LDS images, and all four
+// waves read the B operands of both products from there (16-byte reads for S, transposing reads for O).  The next chunk
+// is on its way into registers while this one is multiplied and goes to the other image afterwards: one workgroup barrier
+// a chunk, one that orders LDS only.  A wave skips the chunks none of its rows sees.
+// ---------------------------------------------------------------------------------------------------------------
+template <int KK>                  // ceil(max(dim, vdim) / 32): 1, 2, 4
+__global__ __launch_bounds__(256) void biased_attn_group_kernel(hxm_biased_attn_args a, int groups_per_seq) {
+  extern __shared__ float lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int G = a.kv_heads, R = a.n_heads / a.kv_heads, D = a.dim, V = a.vdim;
+  const int64_t item = blockIdx.x;                                   // (sequence, kv head, group of four row tiles)
+  const int group = (int)(item % groups_per_seq);
+  const int kvh = (int)((item / groups_per_seq) % G);
+  const int b = (int)(item / ((int64_t)groups_per_seq * G));
+  const int q0 = a.q_cu[b];
+  const int n_rows = (a.q_cu[b + 1] - q0) * R;
+  if (group * 64 >= n_rows) return;                                  // (the whole workgroup: no barrier is left waiting)
+  const int tile = group * 4 + wave;
+  const bool live = tile * 16 < n_rows;                              // a wave past the portion's rows only helps to load
+  const int g = lane >> 4, c = lane & 15;
+  constexpr int RS = 2 * (KK * 32) + 32;                             // bytes per row of an image (a key's columns, padded)
+  constexpr int PR = KK * 4;                                         // 16-byte pieces per row
+  constexpr int NP = (32 * PR + 255) / 256;                          // pieces of a chunk's keys (or values) a thread brings
+  char* base = reinterpret_cast<char*>(lds);
+  char* img_k[2] = {base, base + 32 * RS};
+  char* img_v[2] = {base + 64 * RS, base + 96 * RS};
+  u16* pl = reinterpret_cast<u16*>(base + 128 * RS) + wave * (16 * kPStride);
+  const u16* kc = (const u16*)a.key_cache + (int64_t)kvh * a.head_stride;
+  const u16* vc = (const u16*)a.value_cache + (int64_t)kvh * a.head_stride;
+  const int32_t* table = a.block_table + a.cu_block_lens[b];
+  const u16x8 zero8 = u16x8{0, 0, 0, 0, 0, 0, 0, 0};
+
+  u16x8 qf[KK];
+  {
+    const int r = min(tile * 16 + c, n_rows - 1);
+    const u16* qg = (const u16*)a.q + ((int64_t)(q0 + r / R) * a.n_heads + kvh * R + r % R) * D;
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) {
+      const int col = 32 * kk + 8 * g;
+      qf[kk] = col < D ? *reinterpret_cast<const u16x8*>(qg + col) : zero8;
+    }
+  }
+  int pos[4], lo[4];
+  float slope[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 16 + 4 * g + i;
+    if (r < n_rows) {
+      pos[i] = a.positions[q0 + r / R];
+      lo[i] = first_visible(pos[i], a.mask_kind, a.mask_size);
+      slope[i] = a.slopes ? a.slopes[kvh * R + r % R] : 0.f;
+    } else {
+      pos[i] = -1;      // sees nothing
+      lo[i] = 0;
+      slope[i] = 0.f;
+    }
+  }
+  // rows of a portion are in the order of their positions: the group's first row sees the earliest key, its last the latest
+  const int k_begin = first_visible(a.positions[q0 + (group * 64) / R], a.mask_kind, a.mask_size);
+  const int k_end = a.positions[q0 + min(group * 64 + 63, n_rows - 1) / R];
+  int w_min = 0x7fffffff, w_max = -1;      // the keys this wave's rows see
+  if (live) {
+    w_min = first_visible(a.positions[q0 + (tile * 16) / R], a.mask_kind, a.mask_size);
+    w_max = a.positions[q0 + min(tile * 16 + 15, n_rows - 1) / R];
+  }
+  float m[4], l[4];
+  f32x4 acc[KK * 2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { m[i] = -1.0e30f; l[i] = 0.f; }
+#pragma unroll
+  for (int n = 0; n < KK * 2; ++n) acc[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int bs = a.block_size;
+  const int bshift = (bs & (bs - 1)) == 0 ? __ffs(bs) - 1 : -1;
+  // piece p of a chunk: row p / PR (a key), columns 8 (p % PR) .. + 7
+  u16x8 kr[NP], vr[NP];
+  auto fetch = [&](int key0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int n = 0; n < NP; ++n) {
+      const int p = threadIdx.x + 256 * n;
+      kr[n] = zero8;
+      vr[n] = zero8;
+      if (p < 32 * PR) {
+        const int key = min(key0 + p / PR, k_end), col = (p % PR) * 8;      // (a key past the last one repeats it; masked below)
+        const int page = bshift >= 0 ? key >> bshift : key / bs;
+        const int64_t off = (int64_t)table[page] * a.cache_block_stride + (int64_t)(key - page * bs) * a.cache_row_stride + col;
+        if (col < D) kr[n] = *reinterpret_cast<const u16x8*>(kc + off);
+        if (col < V) vr[n] = *reinterpret_cast<const u16x8*>(vc + off);
+      }
+    }
+  };
+  auto store = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int n = 0; n < NP; ++n) {
+      const int p = threadIdx.x + 256 * n;
+      if (p < 32 * PR) {
+        const int at = (p / PR) * RS + (p % PR) * 16;
+        *reinterpret_cast<u16x8*>(img_k[buf] + at) = kr[n];
+        *reinterpret_cast<u16x8*>(img_v[buf] + at) = vr[n];
+      }
+    }
+  };
+  fetch(k_begin);
+  store(0);
+  lds_barrier();
+  int buf = 0;
+  for (int key0 = k_begin; key0 <= k_end; key0 += 32, buf ^= 1) {
+    const bool more = key0 + 32 <= k_end;
+    if (more) fetch(key0 + 32);
+    if (key0 <= w_max && key0 + 31 >= w_min) {
+      f32x4 sc[2];
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        sc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+          const u16x8 kf = *reinterpret_cast<const u16x8*>(img_k[buf] + (16 * s + c) * RS + (32 * kk + 8 * g) * 2);
+          sc[s] = Mfma<BF16>::mma(qf[kk], kf, sc[s]);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float p[2];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          const int key = key0 + 16 * s + c;
+          const bool seen = key >= lo[i] && key <= pos[i];
+          p[s] = seen ? sc[s][i] * a.scale - slope[i] * (float)(pos[i] - key) : -INFINITY;
+          mx = fmaxf(mx, p[s]);
+        }
+        mx = row16_max(mx);
+        const float m_new = fmaxf(m[i], mx);
+        const float corr = __expf(m[i] - m_new);
+        p[0] = __expf(p[0] - m_new);
+        p[1] = __expf(p[1] - m_new);
+        float ps = p[0] + p[1];
+        ps = row16_sum(ps);
+        l[i] = l[i] * corr + ps;
+        m[i] = m_new;
+#pragma unroll
+        for (int n = 0; n < KK * 2; ++n) acc[n][i] *= corr;
+        pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3)] = BF16::from_float(p[0]);
+        pl[(4 * g + i) * kPStride + 8 * (c >> 2) + (c & 3) + 4] = BF16::from_float(p[1]);
+      }
+      wave_lds_sync();
+      u16x8 pf;
+      {
+        const u16x4 x0 = *reinterpret_cast<const u16x4*>(pl + c * kPStride + 8 * g);
+        const u16x4 x1 = *reinterpret_cast<const u16x4*>(pl + c * kPStride + 8 * g + 4);
+        pf = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+      }
+      const char* vrd = img_v[buf] + (4 * g + (c >> 2)) * RS + (c & 3) * 8;
+#pragma unroll
+      for (int n = 0; n < KK * 2; ++n) {
+        const u16x4 x0 = lds_tr_read(vrd + n * 32);
+        const u16x4 x1 = lds_tr_read(vrd + 16 * RS + n * 32);
+        const u16x8 vv = u16x8{x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        acc[n] = Mfma<BF16>::mma(pf, vv, acc[n]);
+      }
+      wave_lds_sync();      // this wave's reads of P are done before it writes the next chunk's
+    }
+    if (more) store(buf ^ 1);      // (the other image: every wave finished with it before the last barrier)
+    lds_barrier();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 16 + 4 * g + i;
+    if (r >= n_rows) continue;
+    const float inv = 1.0f / l[i];
+    u16* og = (u16*)a.out + ((int64_t)(q0 + r / R) * a.n_heads + kvh * R + r % R) * V;
+#pragma unroll
+    for (int n = 0; n < KK * 2; ++n) {
+      const int col = 16 * n + c;
+      if (col < V) og[col] = BF16::from_float(acc[n][i] * inv);
+    }
+  }
+}
+
 // the splits of a (sequence, kv head, row tile) merged: out = sum_s O_s e^(m_s - M) / sum_s l_s e^(m_s - M)
 __global__ __launch_bounds__(256) void biased_attn_combine_kernel(hxm_biased_attn_args a, int tiles_per_seq) {
   const int64_t item = blockIdx.x;
@@ -428,6 +610,14 @@ int launch_tile(const hxm_biased_attn_args& a, hipStream_t s) {
   const int R = a.n_heads / a.kv_heads;
   const int tiles_per_seq = (int)(((int64_t)a.max_q_len * R + 15) / 16);
   const int n_splits = a.n_splits > 1 ? a.n_splits : 1;
+  if constexpr (KK <= 4) {
+    if (n_splits == 1 && tiles_per_seq >= 4 && a.form != 2) {      // portions of prompts: four row tiles share every chunk
+      const int groups_per_seq = (tiles_per_seq + 3) / 4;
+      const size_t lds_g = (size_t)128 * (2 * (KK * 32) + 32) + 4 * 16 * kPStride * 2;
+      biased_attn_group_kernel<KK><<<dim3((unsigned)((int64_t)a.n_seq * a.kv_heads * groups_per_seq)), dim3(256), lds_g, s>>>(a, groups_per_seq);
+      return hxm::check_launch();
+    }
+  }
   const int64_t items = (int64_t)a.n_seq * a.kv_heads * tiles_per_seq;
   const dim3 grid((unsigned)((items * n_splits + waves - 1) / waves));
   biased_attn_tile_kernel<KK><<<grid, dim3(64 * waves), per_wave * waves, s>>>(a, tiles_per_seq, waves);

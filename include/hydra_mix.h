@@ -241,7 +241,8 @@ typedef struct hxm_biased_attn_args {
   int32_t dtype;
   const int32_t* q_cu;       /* [n_seq + 1]: the tile form's portions */
   int32_t n_seq, max_q_len;  /* max_q_len: the longest portion of the batch (1: every sequence decodes) */
-  int32_t form;              /* 0: the MFMA tile form where it applies (bfloat16, sizes and strides multiples of 8), 1: the row form */
+  int32_t form;              /* 0: the MFMA forms where they apply (bfloat16, sizes and strides multiples of 8), 1: the row form,
+                                2: the MFMA tile form also where the group form (four row tiles sharing each chunk) would run */
   int32_t n_splits;          /* tile form, > 1: a tile's keys are dealt to n_splits waves (<= 64) and merged by a second kernel */
   float* ws_o;               /* n_splits > 1: n_seq * kv_heads * ceil(max_q_len * heads / kv_heads / 16) * n_splits * 16 * ceil16(vdim) floats */
   float* ws_ml;              /* n_splits > 1: ... * n_splits * 32 floats */

@@ -392,7 +392,7 @@ def test_attention_kernel_edges_far_keys_and_page_borders(H, G, D, V, mask, size
         pos = torch.tensor(sum(q_pos, []), dtype=torch.int32, device=DEV)
         tok_seq = torch.tensor(sum([[s] * len(p) for s, p in enumerate(q_pos)], []), dtype=torch.int32, device=DEV)
         q_cu = torch.tensor([0, 40, 73, 74], dtype=torch.int32, device=DEV)
-        for form, max_kv in (("auto", 0), ("auto", 150), ("rows", 0)):      # (with the keys' count known the tile form may split them)
+        for form, max_kv in (("auto", 0), ("auto", 150), ("tile", 0), ("rows", 0)):      # (with the keys' count known the tile form may split them)
             out = biased_attention(q, kc, vc, V, tok_seq, pos, q_cu, table, cu, scale, _dev(slopes), mask, size, max_q_len=40,
                                    kv_heads=G, max_kv_len=max_kv, form=form)
             _close(out, torch.cat(ref), tol, f"attention {mask} {dtype} {form} {max_kv}")
